@@ -1,0 +1,143 @@
+"""``create_attention_mask``: block-sparse attention masks from positions and segment ids.
+
+Host-side mirror of the reference's kvax/ops/mask_creator.py: same function names, arguments,
+defaults and return types (``tuple[AttentionMask, ...]`` of length 1 or 3 whose fields are
+int32 ``[batch, shards, n_outer_blocks]``).  The device work is one call into the C ABI
+(``kvax_mask_build``), which builds all requested masks with two kernel launches.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from kvax_amd import _native
+from kvax_amd.utils.common import (
+    FlashAttentionParamsConfig,
+    get_default_flash_attention_params,
+)
+from kvax_amd.utils.sharding import context_parallel_degree
+from kvax_amd.utils.specs import get_attention_specs
+from kvax_amd.utils.typing import AttentionMask, DeviceArray
+
+
+def _as_ids(x: DeviceArray, name: str) -> torch.Tensor:
+    if x.dim() != 2:
+        raise ValueError(f"{name} must be [batch, seq_len], got shape {tuple(x.shape)}")
+    if not x.is_cuda:
+        raise _native.KvaxNativeError(
+            f"{name} lives on {x.device}: the mask builder only runs on the GPU"
+        )
+    return x.to(torch.int32).contiguous()
+
+
+def build_masks(
+    query_positions: DeviceArray,
+    query_segment_ids: DeviceArray,
+    kv_positions: DeviceArray,
+    kv_segment_ids: DeviceArray,
+    requests: list[tuple[int, int, bool]],
+    skip_pad_tokens: bool = True,
+    num_q_shards: int = 1,
+) -> list[AttentionMask]:
+    """Build one mask per ``(query_block_size, kv_block_size, kv_outer)`` request in one call."""
+    if not 1 <= len(requests) <= _native.KVAX_MAX_MASKS:
+        raise ValueError(f"between 1 and {_native.KVAX_MAX_MASKS} masks per call")
+    q_pos = _as_ids(query_positions, "query_positions")
+    q_seg = _as_ids(query_segment_ids, "query_segment_ids")
+    kv_pos = _as_ids(kv_positions, "kv_positions")
+    kv_seg = _as_ids(kv_segment_ids, "kv_segment_ids")
+    if q_pos.shape != q_seg.shape or kv_pos.shape != kv_seg.shape:
+        raise ValueError("positions and segment ids must have equal shapes")
+    if q_pos.shape[0] != kv_pos.shape[0]:
+        raise ValueError("query and kv batch sizes differ")
+    batch, q_len = q_pos.shape
+    kv_len = kv_pos.shape[1]
+    lib = _native.lib()
+    descs = (_native.MaskDesc * len(requests))()
+    outs = []
+    for d, (qbs, kbs, kv_outer) in zip(descs, requests):
+        n_outer = -(-kv_len // kbs) if kv_outer else -(-q_len // qbs)
+        shards = num_q_shards if kv_outer else 1
+        buf = torch.empty((4, batch, shards, n_outer), dtype=torch.int32, device=q_pos.device)
+        d.query_block_size, d.kv_block_size, d.kv_outer = qbs, kbs, int(kv_outer)
+        d.lower, d.upper = buf[0].data_ptr(), buf[1].data_ptr()
+        d.lower_full, d.upper_full = buf[2].data_ptr(), buf[3].data_ptr()
+        outs.append(buf)
+    ws_bytes = lib.kvax_mask_workspace_bytes(batch, q_len, kv_len, descs, len(requests))
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q_pos.device)
+    stream = torch.cuda.current_stream(q_pos.device).cuda_stream
+    with torch.cuda.device(q_pos.device):
+        rc = lib.kvax_mask_build(
+            q_pos.data_ptr(), q_seg.data_ptr(), kv_pos.data_ptr(), kv_seg.data_ptr(),
+            batch, q_len, kv_len, num_q_shards, int(skip_pad_tokens),
+            descs, len(requests), ws.data_ptr(), ws_bytes, C.c_void_p(stream),
+        )
+    _native.check(rc, "kvax_mask_build")
+    return [AttentionMask(b[0], b[1], b[2], b[3]) for b in outs]
+
+
+def compute_attention_mask(
+    query_positions: DeviceArray,
+    query_segment_ids: DeviceArray,
+    kv_positions: DeviceArray,
+    kv_segment_ids: DeviceArray,
+    kv_block_size: int,
+    query_block_size: int,
+    skip_pad_tokens: bool = True,
+    calculate_dkdv_mask: bool = False,
+    mesh=None,
+) -> AttentionMask:
+    """One mask (kvax/ops/mask_creator.py:338-374)."""
+    get_attention_specs()  # same precondition as the reference: specs must be set
+    return build_masks(
+        query_positions, query_segment_ids, kv_positions, kv_segment_ids,
+        [(query_block_size, kv_block_size, calculate_dkdv_mask)],
+        skip_pad_tokens=skip_pad_tokens, num_q_shards=context_parallel_degree(mesh),
+    )[0]
+
+
+def create_attention_mask(
+    query_positions: DeviceArray,
+    query_segment_ids: DeviceArray,
+    kv_positions: DeviceArray,
+    kv_segment_ids: DeviceArray,
+    fwd_params: FlashAttentionParamsConfig | None = None,
+    bwd_params: FlashAttentionParamsConfig | None = None,
+    calc_bwd_mask: bool = False,
+    skip_pad_tokens: bool = True,
+    mesh=None,
+) -> tuple[AttentionMask, ...]:
+    """Forward mask and, with ``calc_bwd_mask``, the dQ and dK/dV masks.
+
+    Same contract as kvax/ops/mask_creator.py:377-490.  The dQ mask uses the backward block
+    sizes swapped (query blocks of ``bwd_params.kv_block_size``, :459-460); the dK/dV mask has
+    one entry per kv block.  Unlike the reference, ``bwd_params=None`` works (it falls back to
+    the default backward parameters instead of dereferencing None, cf. :454-457).
+    """
+    get_attention_specs()
+    if fwd_params is None:
+        fwd_params = get_default_flash_attention_params(backward=False)
+    requests = [(fwd_params.query_block_size, fwd_params.kv_block_size, False)]
+    if calc_bwd_mask:
+        if bwd_params is None:
+            bwd_params = get_default_flash_attention_params(backward=True)
+        requests.append((bwd_params.kv_block_size, bwd_params.query_block_size, False))
+        requests.append((bwd_params.query_block_size, bwd_params.kv_block_size, True))
+    return tuple(
+        build_masks(
+            query_positions, query_segment_ids, kv_positions, kv_segment_ids, requests,
+            skip_pad_tokens=skip_pad_tokens, num_q_shards=context_parallel_degree(mesh),
+        )
+    )
+
+
+def calculate_mask_sparsity(
+    mask: AttentionMask, query_block_size: int, kv_block_size: int, query_seq_len: int,
+    kv_seq_len: int,
+) -> float:
+    """Fraction of (query block, kv block) pairs inside [lower, upper)
+    (kvax/ops/mask_creator.py:601-625)."""
+    visited = (mask.upper_bounds.long() - mask.lower_bounds.long()).sum().item()
+    batch = mask.lower_bounds.shape[0]
+    return visited / (query_seq_len // query_block_size) / (kv_seq_len // kv_block_size) / batch

@@ -1,0 +1,302 @@
+"""CPU restatement of the reference block-mask builder.  TEST INFRASTRUCTURE ONLY.
+
+Three independent statements of the same function, used to pin each other:
+
+* :func:`block_mask_loop` follows the reference device kernel and its host wrapper step by step
+  (kvax/ops/mask_creator.py:45-152 for the per-outer-block loop, :212-259 for padding and the
+  padding-id remap, :317-333 for the post-processing of "nothing found" sentinels).  Python
+  loops over raw elements: small inputs only.
+* :func:`block_mask_summaries` computes the same thing from per-block (min, max) summaries with
+  numpy; it exists so that 32k-token cases finish in milliseconds.  It is checked against the
+  loop version on random inputs, including the regime (positions restarting per document,
+  unsorted ids) where the heuristic is *not* the dense any/all mask.
+* :func:`block_mask_dense` is the brute-force definition the reference's own test asserts its
+  kernel bit-equal to (tests/test_attention.py:865-905 and :914-1009): build the dense boolean
+  mask, reduce blocks with any/all, take first/last.  Valid as an authority only for the input
+  family that test uses (global ``arange`` positions, contiguous sorted documents, trailing
+  padding, optionally CP-permuted queries).
+
+Parity status: pinned by (1) agreement loop == summaries on random inputs, (2) agreement with
+the dense definition on the reference test's own input family (regenerated exactly: its
+segment lengths come from Python's ``random.seed(0)``, kvax/utils/benchmarking.py:309-324),
+(3) closed forms for a single causal document, (4) invariants.  In the regime where the
+heuristic departs from any/all the step-by-step restatement is the only authority (the
+reference holds no stored vectors and cannot run here).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+PADDING_SEGMENT_ID = -1
+INT32_MAX = np.iinfo(np.int32).max
+
+
+def _pad_inputs(q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size):
+    """mask_creator.py:212-225 -- queries padded with pos -1, kv with INT32_MAX, ids with -1."""
+
+    def pad(pos, seg, block, fill):
+        s = pos.shape[1]
+        sp = (s + block - 1) // block * block
+        if sp != s:
+            pos = np.pad(pos, ((0, 0), (0, sp - s)), constant_values=fill)
+            seg = np.pad(seg, ((0, 0), (0, sp - s)), constant_values=PADDING_SEGMENT_ID)
+        return pos, seg
+
+    q_pos, q_seg = pad(np.asarray(q_pos, np.int32), np.asarray(q_seg, np.int32), query_block_size, -1)
+    kv_pos, kv_seg = pad(
+        np.asarray(kv_pos, np.int32), np.asarray(kv_seg, np.int32), kv_block_size, INT32_MAX
+    )
+    return q_pos, q_seg, kv_pos, kv_seg
+
+
+def _remap_padding(q_seg, kv_seg, kv_len_padded):
+    """mask_creator.py:247-259 -- every -1 becomes ``padded kv length + 1``."""
+    pad_id = kv_len_padded + 1
+    q_seg = np.where(q_seg == PADDING_SEGMENT_ID, pad_id, q_seg).astype(np.int32)
+    kv_seg = np.where(kv_seg == PADDING_SEGMENT_ID, pad_id, kv_seg).astype(np.int32)
+    return q_seg, kv_seg, pad_id
+
+
+def _postprocess(lower, upper, lower_full, upper_full, n_inner, dkdv):
+    """mask_creator.py:317-333."""
+    lower = np.where(lower == n_inner, upper, lower)
+    if dkdv:
+        lower_full = np.where(lower_full == n_inner, upper, lower_full)
+    else:
+        lower_full = np.where(lower_full == n_inner, lower, lower_full)
+    upper_full = np.where(upper_full < lower_full, lower_full, upper_full)
+    return lower, upper, lower_full, upper_full
+
+
+def block_mask_loop(
+    q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size,
+    skip_pad_tokens=True, calculate_dkdv_mask=False,
+):
+    """Element-by-element restatement; returns 4 int32 arrays of shape [B, 1, n_outer]."""
+    q_pos, q_seg, kv_pos, kv_seg = _pad_inputs(
+        q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size
+    )
+    q_seg, kv_seg, pad_id = _remap_padding(q_seg, kv_seg, kv_pos.shape[1])
+    if calculate_dkdv_mask:
+        o_pos, o_seg, i_pos, i_seg = kv_pos, kv_seg, q_pos, q_seg
+        o_bs, i_bs = kv_block_size, query_block_size
+    else:
+        o_pos, o_seg, i_pos, i_seg = q_pos, q_seg, kv_pos, kv_seg
+        o_bs, i_bs = query_block_size, kv_block_size
+    batch = o_pos.shape[0]
+    n_outer = o_pos.shape[1] // o_bs
+    n_inner = i_pos.shape[1] // i_bs
+    out = np.zeros((4, batch, 1, n_outer), np.int32)
+    for b in range(batch):
+        for o in range(n_outer):
+            oseg = o_seg[b, o * o_bs:(o + 1) * o_bs]
+            opos = o_pos[b, o * o_bs:(o + 1) * o_bs]
+            omax_s, omin_s = int(oseg.max()), int(oseg.min())
+            osame = omax_s == omin_s
+            if skip_pad_tokens and osame and omin_s == pad_id:
+                continue  # all four stay 0 (mask_creator.py:69-76)
+            omax_p, omin_p = int(opos.max()), int(opos.min())
+            upper, lower = 0, n_inner
+            upper_full, lower_full = 0, n_inner
+            for i in range(n_inner):
+                iseg = i_seg[b, i * i_bs:(i + 1) * i_bs]
+                ipos = i_pos[b, i * i_bs:(i + 1) * i_bs]
+                imin_s, imax_s = int(iseg.min()), int(iseg.max())
+                isame = imin_s == imax_s
+                seg_overlap = imin_s <= omax_s and omin_s <= imax_s
+                imin_p, imax_p = int(ipos.min()), int(ipos.max())
+                if not calculate_dkdv_mask:  # query is the outer block
+                    attend_pos = omax_p >= imin_p
+                    full_pos = omin_p >= imax_p
+                else:
+                    attend_pos = imax_p >= omin_p
+                    full_pos = imin_p >= omax_p
+                attend = attend_pos and seg_overlap
+                if skip_pad_tokens and imin_s == pad_id:
+                    attend = False
+                if attend:
+                    upper = max(upper, i + 1)
+                    lower = min(lower, i)
+                if osame and isame and full_pos and attend:
+                    upper_full = max(upper_full, i + 1)
+                    lower_full = min(lower_full, i)
+            out[:, b, 0, o] = (lower, upper, lower_full, upper_full)
+    lower, upper, lower_full, upper_full = _postprocess(
+        out[0], out[1], out[2], out[3], n_inner, calculate_dkdv_mask
+    )
+    # the early-exit rows hold lower == 0 != n_inner unless n_inner == 0; nothing to undo
+    return (lower.astype(np.int32), upper.astype(np.int32),
+            lower_full.astype(np.int32), upper_full.astype(np.int32))
+
+
+def block_mask_summaries(
+    q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size,
+    skip_pad_tokens=True, calculate_dkdv_mask=False,
+):
+    """Same function from per-block min/max summaries (vectorised over inner blocks)."""
+    q_pos, q_seg, kv_pos, kv_seg = _pad_inputs(
+        q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size
+    )
+    q_seg, kv_seg, pad_id = _remap_padding(q_seg, kv_seg, kv_pos.shape[1])
+    if calculate_dkdv_mask:
+        o_pos, o_seg, i_pos, i_seg = kv_pos, kv_seg, q_pos, q_seg
+        o_bs, i_bs = kv_block_size, query_block_size
+    else:
+        o_pos, o_seg, i_pos, i_seg = q_pos, q_seg, kv_pos, kv_seg
+        o_bs, i_bs = query_block_size, kv_block_size
+    batch = o_pos.shape[0]
+
+    def summ(x, bs):
+        x = x.reshape(batch, -1, bs)
+        return x.min(-1), x.max(-1)
+
+    os_min, os_max = summ(o_seg, o_bs)
+    op_min, op_max = summ(o_pos, o_bs)
+    is_min, is_max = summ(i_seg, i_bs)
+    ip_min, ip_max = summ(i_pos, i_bs)
+    n_inner = is_min.shape[1]
+    # [B, n_outer, n_inner]
+    seg_overlap = (is_min[:, None, :] <= os_max[:, :, None]) & (os_min[:, :, None] <= is_max[:, None, :])
+    if not calculate_dkdv_mask:
+        attend_pos = op_max[:, :, None] >= ip_min[:, None, :]
+        full_pos = op_min[:, :, None] >= ip_max[:, None, :]
+    else:
+        attend_pos = ip_max[:, None, :] >= op_min[:, :, None]
+        full_pos = ip_min[:, None, :] >= op_max[:, :, None]
+    attend = attend_pos & seg_overlap
+    if skip_pad_tokens:
+        attend &= (is_min != pad_id)[:, None, :]
+    osame = (os_min == os_max)[:, :, None]
+    isame = (is_min == is_max)[:, None, :]
+    full = osame & isame & full_pos & attend
+
+    def first_last(m):
+        any_ = m.any(-1)
+        first = np.where(any_, m.argmax(-1), n_inner)
+        last = np.where(any_, n_inner - m[..., ::-1].argmax(-1), 0)
+        return first, last
+
+    lower, upper = first_last(attend)
+    lower_full, upper_full = first_last(full)
+    if skip_pad_tokens:
+        dead = (os_min == os_max) & (os_min == pad_id)
+        lower = np.where(dead, 0, lower)
+        upper = np.where(dead, 0, upper)
+        lower_full = np.where(dead, 0, lower_full)
+        upper_full = np.where(dead, 0, upper_full)
+    res = _postprocess(lower, upper, lower_full, upper_full, n_inner, calculate_dkdv_mask)
+    return tuple(r.astype(np.int32)[:, None, :] for r in res)
+
+
+def dense_attention_mask(q_pos, q_seg, kv_pos, kv_seg, skip_pad_tokens=True):
+    """[B, Sq, Sk] boolean: same segment and q_pos >= kv_pos (tests/test_attention.py:33-49),
+    minus padding rows/columns when ``skip_pad_tokens`` (:914-924)."""
+    q_pos, q_seg = np.asarray(q_pos), np.asarray(q_seg)
+    kv_pos, kv_seg = np.asarray(kv_pos), np.asarray(kv_seg)
+    m = (q_seg[:, :, None] == kv_seg[:, None, :]) & (q_pos[:, :, None] >= kv_pos[:, None, :])
+    if skip_pad_tokens:
+        m &= (q_seg != PADDING_SEGMENT_ID)[:, :, None]
+        m &= (kv_seg != PADDING_SEGMENT_ID)[:, None, :]
+    return m
+
+
+def _dense_to_bounds(blocks_any, blocks_all, n_inner, kv_mask):
+    """tests/test_attention.py:865-905."""
+    none = ~blocks_any.any(-1)
+    lower = np.where(none, 0, blocks_any.argmax(-1))
+    upper = np.where(none, 0, n_inner - blocks_any[..., ::-1].argmax(-1))
+    none_f = ~blocks_all.any(-1)
+    fallback = upper if kv_mask else lower
+    lower_full = np.where(none_f, fallback, blocks_all.argmax(-1))
+    upper_full = np.where(none_f, fallback, n_inner - blocks_all[..., ::-1].argmax(-1))
+    return tuple(x.astype(np.int32)[:, None, :] for x in (lower, upper, lower_full, upper_full))
+
+
+def block_mask_dense(
+    q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size,
+    skip_pad_tokens=True, calculate_dkdv_mask=False, chunk_tokens=4096,
+):
+    """Brute-force block bounds from the dense mask; sequence lengths must divide the blocks.
+    The dense mask is materialised ``chunk_tokens`` outer rows at a time."""
+    q_pos, q_seg = np.asarray(q_pos), np.asarray(q_seg)
+    kv_pos, kv_seg = np.asarray(kv_pos), np.asarray(kv_seg)
+    b, sq = q_pos.shape
+    sk = kv_pos.shape[1]
+    assert sq % query_block_size == 0 and sk % kv_block_size == 0
+    if calculate_dkdv_mask:
+        o_bs, i_bs, o_len, n_inner = kv_block_size, query_block_size, sk, sq // query_block_size
+    else:
+        o_bs, i_bs, o_len, n_inner = query_block_size, kv_block_size, sq, sk // kv_block_size
+    step = max(o_bs, chunk_tokens // o_bs * o_bs)
+    any_parts, all_parts = [], []
+    for r0 in range(0, o_len, step):
+        sl = slice(r0, min(o_len, r0 + step))
+        if calculate_dkdv_mask:
+            m = dense_attention_mask(q_pos, q_seg, kv_pos[:, sl], kv_seg[:, sl], skip_pad_tokens)
+            m = m.transpose(0, 2, 1)
+        else:
+            m = dense_attention_mask(q_pos[:, sl], q_seg[:, sl], kv_pos, kv_seg, skip_pad_tokens)
+        m = m.reshape(b, m.shape[1] // o_bs, o_bs, n_inner, i_bs)
+        any_parts.append(m.any(axis=(2, 4)))
+        all_parts.append(m.all(axis=(2, 4)))
+    blocks_any = np.concatenate(any_parts, axis=1)
+    blocks_all = np.concatenate(all_parts, axis=1)
+    return _dense_to_bounds(blocks_any, blocks_all, n_inner, calculate_dkdv_mask)
+
+
+def create_attention_mask(
+    q_pos, q_seg, kv_pos, kv_seg, fwd_blocks, bwd_blocks=None, calc_bwd_mask=False,
+    skip_pad_tokens=True, cp=1, impl=block_mask_summaries,
+):
+    """Tuple (fwd,) or (fwd, dq, dkdv) of 4-tuples, mirroring mask_creator.py:377-490.
+
+    ``fwd_blocks`` / ``bwd_blocks`` are (query_block_size, kv_block_size).  The dQ mask swaps the
+    backward block sizes (:459-460).  With ``cp`` > 1 the query axis is cut into ``cp``
+    contiguous shards and every mask is built per shard, as shard_map does with the specs of
+    mask_creator.py:155-178: query-outer masks concatenate along the last axis, the kv-outer mask
+    stacks along axis 1 and holds shard-local query-block indices.
+    """
+    q_pos, q_seg = np.asarray(q_pos, np.int32), np.asarray(q_seg, np.int32)
+    sq = q_pos.shape[1]
+    assert sq % cp == 0
+    ssz = sq // cp
+
+    def build(qbs, kbs, dkdv):
+        parts = [impl(q_pos[:, r * ssz:(r + 1) * ssz], q_seg[:, r * ssz:(r + 1) * ssz],
+                      kv_pos, kv_seg, qbs, kbs, skip_pad_tokens, dkdv) for r in range(cp)]
+        axis = 1 if dkdv else 2
+        return tuple(np.concatenate([p[k] for p in parts], axis=axis) for k in range(4))
+
+    out = [build(fwd_blocks[0], fwd_blocks[1], False)]
+    if calc_bwd_mask:
+        bq, bk = bwd_blocks
+        out.append(build(bk, bq, False))
+        out.append(build(bq, bk, True))
+    return tuple(out)
+
+
+def block_mask_c(
+    q_pos, q_seg, kv_pos, kv_seg, query_block_size, kv_block_size,
+    skip_pad_tokens=True, calculate_dkdv_mask=False,
+):
+    """The C restatement (oracle/mask_oracle.c) through ctypes; build it with ``make -C oracle``."""
+    import ctypes as C
+    from pathlib import Path
+
+    so = Path(__file__).resolve().parent / "libkvax_oracle.so"
+    if not so.exists():
+        raise FileNotFoundError(f"{so} missing: run `make -C oracle`")
+    lib = C.CDLL(str(so))
+    q_pos = np.ascontiguousarray(q_pos, np.int32); q_seg = np.ascontiguousarray(q_seg, np.int32)
+    kv_pos = np.ascontiguousarray(kv_pos, np.int32); kv_seg = np.ascontiguousarray(kv_seg, np.int32)
+    b, sq = q_pos.shape
+    sk = kv_pos.shape[1]
+    n_outer = -(-sk // kv_block_size) if calculate_dkdv_mask else -(-sq // query_block_size)
+    outs = [np.zeros((b, 1, n_outer), np.int32) for _ in range(4)]
+    ptr = lambda a: a.ctypes.data_as(C.c_void_p)
+    rc = lib.kvax_oracle_block_mask(
+        ptr(q_pos), ptr(q_seg), ptr(kv_pos), ptr(kv_seg), b, sq, sk, query_block_size,
+        kv_block_size, int(skip_pad_tokens), int(calculate_dkdv_mask), *map(ptr, outs))
+    if rc != 0:
+        raise ValueError("kvax_oracle_block_mask rejected its arguments")
+    return tuple(outs)
