@@ -69,6 +69,64 @@ int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const int32_t* k
                     int skip_pad_tokens, const kvax_mask_desc* masks, int num_masks,
                     void* workspace, size_t workspace_bytes, kvax_stream_t stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Flash attention, forward and backward.
+ * kvax_fa_fwd replaces the `jt.triton_call` of flash_attention_forward_kernel
+ * (reference kvax/ops/flash_attention_triton.py:1517-1540) and the padding / un-padding around it
+ * (:1457-1472, :1543-1544); kvax_fa_bwd replaces the launches of attn_bwd_preprocess (:1692),
+ * flash_attention_backward_kernel_dquery (:1740), flash_attention_backward_kernel_dkdv (:1778)
+ * or the fused flash_attention_backward_kernel (:1819), and the reduction of dK/dV over the
+ * query heads of a group (:1855-1868).
+ *
+ * Tensors are consumed in the public [batch, seq, heads, head_dim] layout through element
+ * strides {batch, seq, head}; the head_dim axis must be contiguous.  Sequence lengths need not
+ * be multiples of the block sizes: tails are handled inside the kernels.  The reference's
+ * assume_sequential_positions mode (causal test on token indices plus a per-shard offset,
+ * :1421-1451) needs no kernel support: the caller passes those indices as q_pos / kv_pos.
+ * ------------------------------------------------------------------------------------------ */
+typedef struct kvax_fa_args {
+  const void* q;   /* [batch, q_len, num_heads, head_dim]     */
+  const void* k;   /* [batch, kv_len, num_kv_heads, head_dim] */
+  const void* v;   /* [batch, kv_len, num_kv_heads, head_dim] */
+  void* out;       /* forward: output, like q.  backward: input (forward result) */
+  float* lse;      /* [batch, num_heads, q_len] fp32, base-2 log-sum-exp of scale*log2(e)*logits;
+                      forward output / backward input; 0 for rows that attend to nothing */
+  const void* dout; /* backward only: like out */
+  void* dq;         /* backward only: like q, dtype of q */
+  void* dk;         /* backward only: like k, dtype of q */
+  void* dv;         /* backward only: like v, dtype of q */
+  const int32_t* q_pos;  /* [batch, q_len]  */
+  const int32_t* q_seg;  /* [batch, q_len]  */
+  const int32_t* kv_pos; /* [batch, kv_len] */
+  const int32_t* kv_seg; /* [batch, kv_len] */
+  /* block masks as produced by kvax_mask_build: {lower, upper, lower_full, upper_full} */
+  const int32_t* fwd_mask[4];  /* [batch, ceil(q_len / fwd_query_block)], kv blocks of fwd_kv_block */
+  const int32_t* dq_mask[4];   /* [batch, ceil(q_len / bwd_kv_block)], kv blocks of bwd_query_block */
+  const int32_t* dkdv_mask[4]; /* [batch, ceil(kv_len / bwd_kv_block)], query blocks of bwd_query_block */
+  int64_t q_strides[3];
+  int64_t k_strides[3];
+  int64_t v_strides[3];
+  int64_t o_strides[3];
+  int64_t do_strides[3];
+  int64_t dq_strides[3];
+  int64_t dk_strides[3];
+  int64_t dv_strides[3];
+  int32_t batch, q_len, kv_len, num_heads, num_kv_heads, head_dim;
+  int32_t fwd_query_block, fwd_kv_block; /* granularity of fwd_mask */
+  int32_t bwd_query_block, bwd_kv_block; /* granularity of dq_mask (swapped) and dkdv_mask */
+  int32_t dtype;                         /* KVAX_BF16 or KVAX_F16 */
+  int32_t flags;                         /* must be 0 */
+  float scale;
+  int32_t reserved;
+} kvax_fa_args;
+
+size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* args);
+size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* args);
+int kvax_fa_fwd(const kvax_fa_args* args, void* workspace, size_t workspace_bytes,
+                kvax_stream_t stream);
+int kvax_fa_bwd(const kvax_fa_args* args, void* workspace, size_t workspace_bytes,
+                kvax_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

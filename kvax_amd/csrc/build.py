@@ -21,7 +21,7 @@ SOURCES = ["abi.cpp", "mask_builder.hip", "fa_fwd.hip", "fa_bwd.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffast-math",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     f"-I{ROOT / 'include'}", f"-I{CSRC}",

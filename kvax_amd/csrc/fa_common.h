@@ -1,0 +1,123 @@
+// Device-side building blocks shared by the flash-attention kernels (gfx950 only).
+//
+// MFMA operand layouts used throughout (wave64, v_mfma_f32_32x32x16_{bf16,f16}):
+//   A (32 x 16):  lane l holds row  l % 32, k = 8 * (l / 32) + [0, 8)
+//   B (16 x 32):  lane l holds col  l % 32, k = 8 * (l / 32) + [0, 8)
+//   C (32 x 32):  lane l holds col  l % 32, rows 8 * (i / 4) + 4 * (l / 32) + i % 4, i in [0, 16)
+// A C tile can therefore be fed back as a B operand whose contraction index is the C row
+// index: k-slot e of half h in step s (s = 0, 1) is C register 8 * s + e, i.e. row
+// 16 * s + 8 * (e / 4) + 4 * h + e % 4.  The matching A operand gathers those rows with two
+// transposing LDS reads (ds_read_b64_tr_b16), see tr_read_a().
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace kvax {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+#define KVAX_LDS(ptr, T) ((__attribute__((address_space(3))) T*)(ptr))
+
+struct Bf16 {
+  using vec8 = bf16x8;
+  __device__ static __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  __device__ static __forceinline__ float to_float(uint16_t bits) {
+    return __builtin_bit_cast(float, (uint32_t)bits << 16);
+  }
+};
+
+struct F16 {
+  using vec8 = f16x8;
+  __device__ static __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    f16x2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  __device__ static __forceinline__ float to_float(uint16_t bits) {
+    return (float)__builtin_bit_cast(_Float16, bits);
+  }
+};
+
+// Eight consecutive fp32 values -> one 8 x 16-bit MFMA operand.
+template <class Tr>
+__device__ __forceinline__ typename Tr::vec8 pack8(float a0, float a1, float a2, float a3,
+                                                   float a4, float a5, float a6, float a7) {
+  uint4 u = make_uint4(Tr::pack2(a0, a1), Tr::pack2(a2, a3), Tr::pack2(a4, a5), Tr::pack2(a6, a7));
+  return __builtin_bit_cast(typename Tr::vec8, u);
+}
+
+// Transposing LDS read.  Within each group of 16 lanes, lane i passes the address of 4
+// consecutive 16-bit elements; the 16 x 64-bit chunks form a 4 x 16 matrix (row = i / 4, columns
+// 4 * (i % 4) + [0, 4)) and lane i receives column i of it.
+__device__ __forceinline__ s16x4 ds_read_tr16(const void* lds_ptr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(KVAX_LDS(lds_ptr, s16x4));
+}
+
+// A operand (32 x 16) = transpose of a row-major LDS tile X[row][col] (16-bit elements,
+// `stride` bytes per row): A[m][k-slot e] = X[row0 + 8 * (e / 4) + 4 * h + e % 4][col0 + m],
+// the row order that matches a C tile used as B operand (see file header).
+template <class Tr>
+__device__ __forceinline__ typename Tr::vec8 tr_read_a(const char* tile, int stride, int row0,
+                                                       int col0, int lane) {
+  const int g = lane >> 4, i = lane & 15;
+  const int h = g >> 1;
+  const char* p = tile + (row0 + 4 * h + (i >> 2)) * stride + (col0 + 16 * (g & 1) + 4 * (i & 3)) * 2;
+  s16x4 lo = ds_read_tr16(p);
+  s16x4 hi = ds_read_tr16(p + 8 * stride);
+  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(typename Tr::vec8, v);
+}
+
+// Same gather but with the natural k order (k-slot e of half h = row row0 + 8 * h + e): used when
+// the B operand comes from memory rather than from a C tile.
+template <class Tr>
+__device__ __forceinline__ typename Tr::vec8 tr_read_a_linear(const char* tile, int stride,
+                                                              int row0, int col0, int lane) {
+  const int g = lane >> 4, i = lane & 15;
+  const int h = g >> 1;
+  const char* p = tile + (row0 + 8 * h + (i >> 2)) * stride + (col0 + 16 * (g & 1) + 4 * (i & 3)) * 2;
+  s16x4 lo = ds_read_tr16(p);
+  s16x4 hi = ds_read_tr16(p + 4 * stride);
+  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(typename Tr::vec8, v);
+}
+
+// Natural operand read: 8 consecutive elements of row `row` starting at column `col`.
+template <class Tr>
+__device__ __forceinline__ typename Tr::vec8 read_row8(const char* tile, int stride, int row,
+                                                       int col) {
+  return *reinterpret_cast<const typename Tr::vec8*>(tile + row * stride + col * 2);
+}
+
+// v_exp_f32 / v_log_f32 without the denormal-range fix-ups of exp2f / log2f.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32); }
+
+// Work-group index -> work item, so that each XCD (work-groups are dealt round-robin to the 8
+// XCDs) walks a contiguous range of items and neighbouring items share that XCD's L2.
+__device__ __forceinline__ int xcd_contiguous(int linear, int total) {
+  constexpr int kXcds = 8;
+  const int per = total / kXcds, rem = total % kXcds;
+  const int xcd = linear % kXcds, idx = linear / kXcds;
+  return xcd * per + (xcd < rem ? xcd : rem) + idx;
+}
+
+}  // namespace kvax

@@ -1,0 +1,454 @@
+// Flash-attention forward for gfx950 (FA2 online softmax, block-sparse document mask, GQA).
+//
+// Semantics: reference kvax/ops/flash_attention_triton.py:57-370 (three kv ranges per query
+// block taken from the block mask: [lower, lower_full) and [upper_full, upper) apply the element
+// mask, [lower_full, upper_full) is mask-free; base-2 online softmax with scale*log2(e) folded
+// in; P rounded to the input dtype before P.V; lse = m + log2(l)).  Differences, all inside
+// what the reference's tests treat as don't-care: padding tokens (segment id -1) attend to
+// nothing and rows without any attendable key produce exact zeros (and lse 0).
+//
+// Design (not the reference's): the wavefront computes S^T = K Q^T so that each lane owns one
+// query column of the 32x32 MFMA result.  Row max / row sum are then in-lane reductions plus a
+// single exchange between the two half-waves, and the exponentiated tile is already in the
+// B-operand layout of the second contraction O^T += V^T P^T -- P never goes through LDS.  V^T
+// operands are gathered from the row-major V tile with transposing LDS reads.  K/V tiles are
+// staged through LDS once per work-group (double buffered, prefetched through registers) and
+// shared by the work-group's wavefronts; the query heads of one GQA group run as neighbouring
+// work-groups on one XCD so K/V tiles are served from that XCD's L2.
+#include "common.h"
+#include "fa_common.h"
+
+namespace kvax {
+namespace {
+
+constexpr int kTK = 64;  // kv rows per LDS tile
+
+struct FwdParams {
+  const char* q;
+  const char* k;
+  const char* v;
+  char* out;
+  float* lse;
+  const int32_t* q_pos;
+  const int32_t* q_seg;
+  const int32_t* kv_pos;
+  const int32_t* kv_seg;
+  const int32_t* lower;
+  const int32_t* upper;
+  const int32_t* lower_full;
+  const int32_t* upper_full;
+  int64_t q_sb, q_ss, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  int batch, q_len, kv_len, num_heads, num_kv_heads, group;
+  int qbs, kbs, n_qblocks;
+  int num_q_tiles, total_items;
+  float scale_log2;
+};
+
+template <int D>
+struct FwdSmem {
+  static constexpr int kKStride = D * 2 + 16;  // bytes; 16 B pad => conflict-free b128 row reads
+  static constexpr int kVStride = D * 2 + 64;  // bytes; 64 B pad spreads the 4-row tr reads
+  static constexpr int kKBytes = kTK * kKStride;
+  static constexpr int kVBytes = kTK * kVStride;
+  static constexpr int kIdBytes = 2 * kTK * 4;  // seg + pos
+  static constexpr int kStage = kKBytes + kVBytes + kIdBytes;
+  static constexpr int kTotal = 2 * kStage;
+};
+
+// Cooperative global -> register -> LDS staging of one K/V tile (+ its ids).
+template <int D, int NT>
+struct TileLoader {
+  static constexpr int kChunksPerRow = D / 8;                    // 16-byte chunks
+  static constexpr int kPerThread = kTK * kChunksPerRow / NT;    // chunks per thread per tensor
+  static_assert(kTK * kChunksPerRow % NT == 0, "tile must split evenly over the work-group");
+  uint4 kreg[kPerThread];
+  uint4 vreg[kPerThread];
+  int32_t idreg;
+
+  __device__ __forceinline__ void load(const FwdParams& p, const char* kbase, const char* vbase,
+                                       const int32_t* seg, const int32_t* pos, int kv0, int tid) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) {
+      const int id = tid + i * NT;
+      const int row = id / kChunksPerRow, ch = id % kChunksPerRow;
+      const int kv = kv0 + row;
+      if (kv < p.kv_len) {
+        kreg[i] = *reinterpret_cast<const uint4*>(kbase + (int64_t)kv * p.k_ss * 2 + ch * 16);
+        vreg[i] = *reinterpret_cast<const uint4*>(vbase + (int64_t)kv * p.v_ss * 2 + ch * 16);
+      } else {
+        kreg[i] = make_uint4(0, 0, 0, 0);
+        vreg[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+    if (tid < 2 * kTK) {
+      const int kv = kv0 + (tid % kTK);
+      const bool is_seg = tid < kTK;
+      idreg = is_seg ? -1 : 0;
+      if (kv < p.kv_len) idreg = is_seg ? seg[kv] : pos[kv];
+    }
+  }
+
+  __device__ __forceinline__ void store(char* stage, int tid) {
+    char* kt = stage;
+    char* vt = stage + FwdSmem<D>::kKBytes;
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) {
+      const int id = tid + i * NT;
+      const int row = id / kChunksPerRow, ch = id % kChunksPerRow;
+      *reinterpret_cast<uint4*>(kt + row * FwdSmem<D>::kKStride + ch * 16) = kreg[i];
+      *reinterpret_cast<uint4*>(vt + row * FwdSmem<D>::kVStride + ch * 16) = vreg[i];
+    }
+    if (tid < 2 * kTK)
+      reinterpret_cast<int32_t*>(stage + FwdSmem<D>::kKBytes + FwdSmem<D>::kVBytes)[tid] = idreg;
+  }
+};
+
+// One work-group: NW wavefronts x (32 * MQ) query rows of one (batch, head); loops over kv tiles.
+template <class Tr, int D, int MQ, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
+  using vec8 = typename Tr::vec8;
+  using Smem = FwdSmem<D>;
+  constexpr int NT = NW * 64;
+  constexpr int TQ = NW * 32 * MQ;
+  constexpr int KSTEPS = D / 16;  // contraction steps of S^T = K Q^T
+  constexpr int DT = D / 32;      // 32-row tiles of O^T
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int c = lane % 32, h = lane / 32;
+
+  // ---- work item: heads of a GQA group adjacent, long (late) query tiles first -------------
+  int item = xcd_contiguous(blockIdx.x, p.total_items);
+  const int g = item % p.group;
+  item /= p.group;
+  const int q_tile = p.num_q_tiles - 1 - item % p.num_q_tiles;
+  item /= p.num_q_tiles;
+  const int kv_head = item % p.num_kv_heads;
+  const int b = item / p.num_kv_heads;
+  const int head = kv_head * p.group + g;
+  const int q0 = q_tile * TQ;
+
+  const int32_t* q_seg = p.q_seg + (int64_t)b * p.q_len;
+  const int32_t* q_pos = p.q_pos + (int64_t)b * p.q_len;
+  const int32_t* kv_seg = p.kv_seg + (int64_t)b * p.kv_len;
+  const int32_t* kv_pos = p.kv_pos + (int64_t)b * p.kv_len;
+  const char* qbase = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2;
+  const char* kbase = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh) * 2;
+  const char* vbase = p.v + ((int64_t)b * p.v_sb + (int64_t)kv_head * p.v_sh) * 2;
+  char* obase = p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh) * 2;
+  float* lse = p.lse + ((int64_t)b * p.num_heads + head) * p.q_len;
+
+  // ---- kv range of the work-group: union over the mask's query blocks it covers ------------
+  // (element units; the "full" range is the intersection)
+  int lo = 0x7fffffff, hi = 0, flo = 0, fhi = 0x7fffffff;
+  int min_hi = 0x7fffffff, max_lo = 0;
+  {
+    const int qb0 = q0 / p.qbs;
+    const int qb1 = min((q0 + TQ - 1) / p.qbs, p.n_qblocks - 1);
+    for (int qb = qb0; qb <= qb1; qb++) {
+      const int64_t mi = (int64_t)b * p.n_qblocks + qb;
+      const int l_ = p.lower[mi] * p.kbs, u_ = p.upper[mi] * p.kbs;
+      const int lf = p.lower_full[mi] * p.kbs, uf = p.upper_full[mi] * p.kbs;
+      flo = max(flo, lf);
+      fhi = min(fhi, uf);
+      if (u_ > l_) {
+        lo = min(lo, l_);
+        hi = max(hi, u_);
+        min_hi = min(min_hi, u_);
+        max_lo = max(max_lo, l_);
+      } else {
+        min_hi = 0;  // a block that attends to nothing: every tile needs the range test
+        max_lo = 0x7fffffff;
+      }
+    }
+  }
+  hi = min(hi, p.kv_len);
+  const int t_lo = lo / kTK;
+  const int t_hi = hi > lo ? (hi + kTK - 1) / kTK : t_lo;
+  const int tf_lo = (flo + kTK - 1) / kTK, tf_hi = fhi / kTK;
+
+  // ---- per-lane query columns ------------------------------------------------------------
+  int qrow[MQ], qseg[MQ], qpos[MQ], col_lo[MQ], col_hi[MQ];
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    qrow[qt] = q0 + (wave * MQ + qt) * 32 + c;
+    const bool in = qrow[qt] < p.q_len;
+    qseg[qt] = in ? q_seg[qrow[qt]] : -1;
+    qpos[qt] = in ? q_pos[qrow[qt]] : 0;
+    col_lo[qt] = col_hi[qt] = 0;
+    if (in && qseg[qt] != -1) {
+      const int64_t mi = (int64_t)b * p.n_qblocks + qrow[qt] / p.qbs;
+      col_lo[qt] = p.lower[mi] * p.kbs;
+      col_hi[qt] = p.upper[mi] * p.kbs;
+    }
+  }
+
+  f32x16 o[DT][MQ];
+  float m_run[MQ], l_run[MQ];
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    m_run[qt] = -1e30f;
+    l_run[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) o[dt][qt][i] = 0.f;
+  }
+
+  if (t_hi > t_lo) {
+    // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step
+    vec8 qf[MQ][KSTEPS];
+#pragma unroll
+    for (int qt = 0; qt < MQ; qt++) {
+      const bool in = qrow[qt] < p.q_len;
+      const char* row = qbase + (int64_t)(in ? qrow[qt] : 0) * p.q_ss * 2;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        uint4 u = make_uint4(0, 0, 0, 0);
+        if (in) u = *reinterpret_cast<const uint4*>(row + (16 * ks + 8 * h) * 2);
+        qf[qt][ks] = __builtin_bit_cast(vec8, u);
+      }
+    }
+
+    TileLoader<D, NT> loader;
+    loader.load(p, kbase, vbase, kv_seg, kv_pos, t_lo * kTK, tid);
+    loader.store(smem, tid);
+    __syncthreads();
+
+    for (int t = t_lo; t < t_hi; t++) {
+      const int kv0 = t * kTK;
+      char* stage = smem + ((t - t_lo) & 1) * Smem::kStage;
+      char* next_stage = smem + ((t - t_lo + 1) & 1) * Smem::kStage;
+      const bool has_next = t + 1 < t_hi;
+      if (has_next) loader.load(p, kbase, vbase, kv_seg, kv_pos, kv0 + kTK, tid);
+
+      const char* ktile = stage;
+      const char* vtile = stage + Smem::kKBytes;
+      const int32_t* ids = reinterpret_cast<const int32_t*>(stage + Smem::kKBytes + Smem::kVBytes);
+
+      // ---- S^T = K Q^T -------------------------------------------------------------------
+      f32x16 s[2][MQ];
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) s[kt][qt][i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        vec8 a[2];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+          a[kt] = read_row8<Tr>(ktile, Smem::kKStride, 32 * kt + c, 16 * ks + 8 * h);
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+          for (int qt = 0; qt < MQ; qt++) s[kt][qt] = Tr::mfma(a[kt], qf[qt][ks], s[kt][qt]);
+      }
+
+      // ---- scale, element mask ------------------------------------------------------------
+      const bool full = t >= tf_lo && t < tf_hi;
+      const bool range_test = kv0 < max_lo || kv0 + kTK > min_hi;
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) s[kt][qt][i] *= p.scale_log2;
+        if (!full) {
+#pragma unroll
+          for (int g4 = 0; g4 < 4; g4++) {
+            const int r0 = 32 * kt + 8 * g4 + 4 * h;
+            const int4 ksg = *reinterpret_cast<const int4*>(ids + r0);
+            const int4 kps = *reinterpret_cast<const int4*>(ids + kTK + r0);
+            const int sg[4] = {ksg.x, ksg.y, ksg.z, ksg.w};
+            const int ps[4] = {kps.x, kps.y, kps.z, kps.w};
+#pragma unroll
+            for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                bool ok = (sg[j] == qseg[qt]) && (qpos[qt] >= ps[j]);
+                if (range_test) {
+                  const int kv = kv0 + r0 + j;
+                  ok = ok && kv >= col_lo[qt] && kv < col_hi[qt];
+                } else {
+                  ok = ok && col_hi[qt] > 0;
+                }
+                if (!ok) s[kt][qt][4 * g4 + j] = -INFINITY;
+              }
+          }
+        }
+      }
+
+      // ---- online softmax (per query column = per lane, halves combined once) --------------
+      vec8 pb[2][2][MQ];
+#pragma unroll
+      for (int qt = 0; qt < MQ; qt++) {
+        float mx = s[0][qt][0];
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
+        mx = fmaxf(mx, xor32(mx));
+        const float m_new = fmaxf(m_run[qt], mx);
+        if (__any(m_new > m_run[qt])) {
+          const float alpha = fast_exp2(m_run[qt] - m_new);
+          l_run[qt] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
+        }
+        m_run[qt] = m_new;
+        float sum = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+          for (int i = 0; i < 16; i++) {
+            const float e = fast_exp2(s[kt][qt][i] - m_new);
+            s[kt][qt][i] = e;
+            sum += e;
+          }
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+            pb[kt][st][qt] = pack8<Tr>(s[kt][qt][8 * st + 0], s[kt][qt][8 * st + 1],
+                                       s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3],
+                                       s[kt][qt][8 * st + 4], s[kt][qt][8 * st + 5],
+                                       s[kt][qt][8 * st + 6], s[kt][qt][8 * st + 7]);
+        }
+        l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
+      }
+
+      // ---- O^T += V^T P^T -----------------------------------------------------------------
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++) {
+            const vec8 a = tr_read_a<Tr>(vtile, Smem::kVStride, 32 * kt + 16 * st, 32 * dt, lane);
+#pragma unroll
+            for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
+          }
+
+      if (has_next) loader.store(next_stage, tid);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue: normalise, write O (query dtype) and lse --------------------------------
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    const float l = l_run[qt] + xor32(l_run[qt]);
+    const bool alive = l > 0.f && col_hi[qt] > 0;  // padding / out-of-range rows stay zero
+    const float inv = alive ? 1.f / l : 0.f;
+    if (qrow[qt] < p.q_len) {
+      char* row = obase + (int64_t)qrow[qt] * p.o_ss * 2;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          uint2 u;
+          u.x = Tr::pack2(o[dt][qt][4 * g4 + 0] * inv, o[dt][qt][4 * g4 + 1] * inv);
+          u.y = Tr::pack2(o[dt][qt][4 * g4 + 2] * inv, o[dt][qt][4 * g4 + 3] * inv);
+          *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
+        }
+      if (h == 0) lse[qrow[qt]] = alive ? m_run[qt] + fast_log2(l) : 0.f;
+    }
+  }
+}
+
+template <class Tr, int D, int MQ, int NW>
+int launch_fwd(const FwdParams& p0, hipStream_t stream) {
+  FwdParams p = p0;
+  constexpr int TQ = NW * 32 * MQ;
+  p.num_q_tiles = cdiv(p.q_len, TQ);
+  p.total_items = p.batch * p.num_heads * p.num_q_tiles;
+  if (p.total_items == 0) return KVAX_OK;
+  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW>;
+  constexpr int smem = FwdSmem<D>::kTotal;
+  static bool configured = false;  // benign race: the attribute is idempotent
+  if (!configured) {
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem) !=
+        hipSuccess)
+      return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for the forward kernel", smem);
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
+  return check_launch("fa_fwd_kernel");
+}
+
+}  // namespace
+
+int validate_fa_common(const kvax_fa_args* a) {
+  if (!a) return fail(KVAX_EINVAL, "args is null");
+  if (a->batch < 0 || a->q_len < 0 || a->kv_len < 0 || a->num_heads <= 0 || a->num_kv_heads <= 0)
+    return fail(KVAX_EINVAL, "bad batch/length/head counts");
+  if (a->num_heads % a->num_kv_heads)
+    return fail(KVAX_EINVAL, "num_heads %d is not a multiple of num_kv_heads %d", a->num_heads,
+                a->num_kv_heads);
+  if (a->head_dim != 64 && a->head_dim != 128)
+    return fail(KVAX_EUNSUPPORTED, "head_dim %d is not built (64 and 128 are)", a->head_dim);
+  if (a->dtype != KVAX_BF16 && a->dtype != KVAX_F16)
+    return fail(KVAX_EUNSUPPORTED, "dtype %d is not supported (bf16 and f16 are)", a->dtype);
+  if (a->flags != 0) return fail(KVAX_EINVAL, "flags must be 0");
+  if (!a->q || !a->k || !a->v || !a->out || !a->lse || !a->q_pos || !a->q_seg || !a->kv_pos ||
+      !a->kv_seg)
+    return fail(KVAX_EINVAL, "null tensor pointer");
+  const int64_t* strides[] = {a->q_strides, a->k_strides, a->v_strides, a->o_strides};
+  for (auto s : strides)
+    for (int i = 0; i < 3; i++)
+      if (s[i] % 8) return fail(KVAX_EINVAL, "strides must be multiples of 8 elements (16 bytes)");
+  const void* ptrs[] = {a->q, a->k, a->v, a->out};
+  for (auto ptr : ptrs)
+    if ((uintptr_t)ptr % 16) return fail(KVAX_EINVAL, "tensor pointers must be 16-byte aligned");
+  return KVAX_OK;
+}
+
+}  // namespace kvax
+
+using namespace kvax;
+
+extern "C" size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args*) { return 0; }
+
+extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void*, size_t, kvax_stream_t stream_) {
+  if (int rc = validate_fa_common(a)) return rc;
+  if (a->fwd_query_block <= 0 || a->fwd_kv_block <= 0)
+    return fail(KVAX_EINVAL, "forward block sizes must be positive");
+  for (int i = 0; i < 4; i++)
+    if (!a->fwd_mask[i]) return fail(KVAX_EINVAL, "forward mask is missing");
+  FwdParams p{};
+  p.q = (const char*)a->q;
+  p.k = (const char*)a->k;
+  p.v = (const char*)a->v;
+  p.out = (char*)a->out;
+  p.lse = a->lse;
+  p.q_pos = a->q_pos;
+  p.q_seg = a->q_seg;
+  p.kv_pos = a->kv_pos;
+  p.kv_seg = a->kv_seg;
+  p.lower = a->fwd_mask[0];
+  p.upper = a->fwd_mask[1];
+  p.lower_full = a->fwd_mask[2];
+  p.upper_full = a->fwd_mask[3];
+  p.q_sb = a->q_strides[0], p.q_ss = a->q_strides[1], p.q_sh = a->q_strides[2];
+  p.k_sb = a->k_strides[0], p.k_ss = a->k_strides[1], p.k_sh = a->k_strides[2];
+  p.v_sb = a->v_strides[0], p.v_ss = a->v_strides[1], p.v_sh = a->v_strides[2];
+  p.o_sb = a->o_strides[0], p.o_ss = a->o_strides[1], p.o_sh = a->o_strides[2];
+  p.batch = a->batch, p.q_len = a->q_len, p.kv_len = a->kv_len;
+  p.num_heads = a->num_heads, p.num_kv_heads = a->num_kv_heads;
+  p.group = a->num_heads / a->num_kv_heads;
+  p.qbs = a->fwd_query_block, p.kbs = a->fwd_kv_block;
+  p.n_qblocks = cdiv(a->q_len, a->fwd_query_block);
+  p.scale_log2 = a->scale * 1.4426950408889634f;
+  hipStream_t stream = (hipStream_t)stream_;
+  if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
+  const bool bf16 = a->dtype == KVAX_BF16;
+  if (a->head_dim == 128)
+    return bf16 ? launch_fwd<Bf16, 128, 1, 4>(p, stream) : launch_fwd<F16, 128, 1, 4>(p, stream);
+  return bf16 ? launch_fwd<Bf16, 64, 1, 4>(p, stream) : launch_fwd<F16, 64, 1, 4>(p, stream);
+}

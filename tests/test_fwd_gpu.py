@@ -1,0 +1,172 @@
+"""Forward parity of the HIP flash-attention kernel (through the C ABI) with the dense CPU oracle.
+
+Tolerance: max abs error <= 2e-2 on O over all rows (padding rows must be exactly zero), the
+bound the reference's forward tests use (kvax/utils/benchmarking.py:601-609) and the one the
+build's target states.
+"""
+import numpy as np
+import pytest
+import torch
+
+from kvax_amd import create_attention_mask, flash_attention
+from kvax_amd.utils import FlashAttentionParamsConfig, attention_specs
+from kvax_amd.utils.benchmarking import (
+    generate_random_segments_lengths,
+    make_random_attention_inputs,
+    workload,
+)
+from oracle import attention_oracle as ao
+
+pytestmark = pytest.mark.gpu
+TP_SPECS = (("data", None, "model", None), ("data", None, "model", None))
+ATOL = 2e-2
+
+
+def run_forward(data, scale, qbs, kbs, calc_bwd=False, bwd=None):
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    params = FlashAttentionParamsConfig(query_block_size=qbs, kv_block_size=kbs)
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg, fwd_params=params,
+                                     bwd_params=bwd, calc_bwd_mask=calc_bwd)
+        out = flash_attention(q, k, v, q_pos, q_seg, kv_pos, kv_seg, mask, scale=scale,
+                              fwd_params=params, bwd_params=bwd)
+    return out
+
+
+def oracle_forward(data, scale, heads=None):
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = [x.cpu() for x in data]
+    out, _ = ao.attention_forward(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                  q_pos.numpy(), q_seg.numpy(), kv_pos.numpy(), kv_seg.numpy(),
+                                  scale, dtype=np.float64, heads=heads)
+    return out
+
+
+def check(out, ref, q_seg, heads=None):
+    out = out.float().cpu().numpy()
+    assert np.isfinite(out).all()
+    if heads is not None:
+        out, ref = out[:, :, heads], ref[:, :, heads]
+    err = np.abs(out - ref).max()
+    assert err <= ATOL, f"max abs err {err:.4g}"
+    pad = q_seg.cpu().numpy() == -1
+    assert (out[pad] == 0).all(), "padding query rows must be exactly zero"
+
+
+# (q_len, kv_len, heads, kv_heads, head_dim, pad, segments, qbs, kbs): the shape families of the
+# reference's forward tests (tests/test_attention.py:304-341) at the head dims built here
+CASES = [
+    (384, 384, 8, 8, 64, 0, 1, 64, 64),
+    (400, 400, 8, 8, 64, 0, 1, 64, 64),
+    (384, 256, 8, 8, 64, 0, 1, 64, 64),
+    (384, 300, 4, 4, 128, 0, 1, 64, 64),
+    (400, 256, 4, 4, 128, 0, 1, 128, 128),
+    (400, 300, 4, 4, 128, 0, 1, 128, 64),
+    (256, 1, 8, 8, 64, 0, 1, 64, 64),
+    (300, 1, 4, 4, 128, 0, 1, 64, 64),
+    (384, 384, 8, 8, 128, 100, 1, 64, 64),
+    (384, 384, 8, 8, 128, 383, 1, 64, 64),
+    (384, 384, 16, 8, 128, 0, 1, 128, 128),
+    (384, 384, 16, 1, 64, 100, 1, 64, 128),
+    (1024, 1024, 8, 2, 128, 77, 5, 128, 128),
+    (1024, 1024, 8, 2, 128, 0, 12, 64, 64),
+    (2048, 2048, 4, 4, 64, 300, 7, 128, 128),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16])
+def test_forward_matches_dense_oracle(device, case, dtype):
+    sq, sk, hq, hkv, d, pad, nseg, qbs, kbs = case
+    lengths = generate_random_segments_lengths(min(sq, sk), nseg)
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d, d, seed=sq + sk + d,
+                                               num_pad_tokens=min(pad, sk - 1),
+                                               list_of_segment_lengths=lengths, dtype=dtype,
+                                               device=device)
+    out = run_forward(data, scale, qbs, kbs)
+    check(out, oracle_forward(data, scale), data[4])
+
+
+def test_forward_fp16(device):
+    data, scale = make_random_attention_inputs(1, 512, 512, 4, 2, 128, 128, seed=3,
+                                               num_pad_tokens=50, dtype=torch.float16, device=device)
+    out = run_forward(data, scale, 128, 128)
+    check(out, oracle_forward(data, scale), data[4])
+
+
+@pytest.mark.parametrize("kv_len, start", [(384, 300), (512, 500), (500, 300), (4096, (1200, 200, 1000, 3500))])
+def test_decode_single_query(device, kv_len, start):
+    """q_len = 1 with per-row start positions (tests/test_attention.py:1089-1128)."""
+    data, scale = make_random_attention_inputs(4, 1, kv_len, 16, 8, 128, 128, seed=kv_len,
+                                               start_query_position=start, device=device)
+    out = run_forward(data, scale, 64, 64)
+    check(out, oracle_forward(data, scale), data[4])
+
+
+def test_positions_restart_per_document(device):
+    """cpu_plumbing layout (positions restart, padding tail) in bf16 on the GPU."""
+    w = workload("cpu_plumbing")
+    w.dtype = torch.bfloat16
+    q, k, v = w.draw_tensors(0, device, with_dout=False)
+    data = (q, k, v) + w.ids(device)
+    out = run_forward(data, w.scale, 64, 64)
+    check(out, oracle_forward(data, w.scale), data[4])
+
+
+def test_packed_documents_equal_separate_runs(device):
+    """Document masking == block-diagonal concatenation of independent causal attentions."""
+    lengths = [200, 56, 312, 200]
+    data, scale = make_random_attention_inputs(1, 768, 768, 4, 2, 128, 128, seed=11,
+                                               list_of_segment_lengths=lengths, device=device)
+    packed = run_forward(data, scale, 64, 64)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    at = 0
+    for n in lengths:
+        sl = slice(at, at + n)
+        part = (q[:, sl].contiguous(), k[:, sl].contiguous(), v[:, sl].contiguous(),
+                q_pos[:, sl] - at, torch.zeros_like(q_seg[:, sl]), kv_pos[:, sl] - at,
+                torch.zeros_like(kv_seg[:, sl]))
+        single = run_forward(part, scale, 64, 64)
+        # tiles align differently in the two runs, so sums round differently: allow one bf16
+        # ulp of an O(1) value
+        assert (packed[:, sl].float() - single.float()).abs().max().item() <= 1.6e-2
+        at += n
+
+
+def test_constant_positions_are_bidirectional(device):
+    data, scale = make_random_attention_inputs(1, 256, 256, 2, 2, 64, 64, seed=5, device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    data = (q, k, v, torch.zeros_like(q_pos), q_seg, torch.zeros_like(kv_pos), kv_seg)
+    out = run_forward(data, scale, 64, 64).float().cpu()
+    s = torch.einsum("bqhd,bkhd->bhqk", q.float().cpu(), k.float().cpu()) * scale
+    ref = torch.einsum("bhqk,bkhd->bqhd", s.softmax(-1), v.float().cpu())
+    assert (out - ref).abs().max().item() <= ATOL
+
+
+@pytest.mark.parametrize("name, heads", [("dense_causal", [0, 13]), ("doc32k", [5]),
+                                         ("block_skip", [0, 63])])
+def test_measurement_workloads_sampled_heads(device, name, heads):
+    """Full-size configurations; the dense oracle is evaluated for a sample of heads only."""
+    w = workload(name)
+    q, k, v = w.draw_tensors(0, device, with_dout=False)
+    data = (q, k, v) + w.ids(device)
+    out = run_forward(data, w.scale, *w.fwd_blocks)
+    b = slice(0, 1)  # first batch row is enough for the oracle
+    small = tuple(x[b] for x in data)
+    q_, k_, v_, q_pos, q_seg, kv_pos, kv_seg = [x.cpu() for x in small]
+    ref, _ = ao.attention_forward(q_.float().numpy(), k_.float().numpy(), v_.float().numpy(),
+                                  q_pos.numpy(), q_seg.numpy(), kv_pos.numpy(), kv_seg.numpy(),
+                                  w.scale, dtype=np.float32, heads=heads, row_block=2048)
+    check(out[b], ref, q_seg, heads=heads)
+
+
+def test_errors(device):
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 64, 64, device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg)
+        with pytest.raises(NotImplementedError):
+            flash_attention(*data, mask, bias=torch.zeros(1, device=device))
+        with pytest.raises(ValueError):
+            flash_attention(*data, ())
+        with pytest.raises(ValueError):
+            flash_attention(q[..., :48], k[..., :48], v[..., :48], q_pos, q_seg, kv_pos, kv_seg, mask)
