@@ -84,6 +84,11 @@ int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const int32_t* k
  * assume_sequential_positions mode (causal test on token indices plus a per-shard offset,
  * :1421-1451) needs no kernel support: the caller passes those indices as q_pos / kv_pos.
  * ------------------------------------------------------------------------------------------ */
+enum {
+  KVAX_FA_DKDV_F32 = 1 /* backward writes dk / dv as fp32 (the reference kernels' output type,
+                          flash_attention_triton.py:1729-1730) instead of the dtype of q */
+};
+
 typedef struct kvax_fa_args {
   const void* q;   /* [batch, q_len, num_heads, head_dim]     */
   const void* k;   /* [batch, kv_len, num_kv_heads, head_dim] */
@@ -93,8 +98,8 @@ typedef struct kvax_fa_args {
                       forward output / backward input; 0 for rows that attend to nothing */
   const void* dout; /* backward only: like out */
   void* dq;         /* backward only: like q, dtype of q */
-  void* dk;         /* backward only: like k, dtype of q */
-  void* dv;         /* backward only: like v, dtype of q */
+  void* dk;         /* backward only: like k; dtype of q, or fp32 with KVAX_FA_DKDV_F32 */
+  void* dv;         /* backward only: like v; dtype of q, or fp32 with KVAX_FA_DKDV_F32 */
   const int32_t* q_pos;  /* [batch, q_len]  */
   const int32_t* q_seg;  /* [batch, q_len]  */
   const int32_t* kv_pos; /* [batch, kv_len] */
@@ -115,7 +120,7 @@ typedef struct kvax_fa_args {
   int32_t fwd_query_block, fwd_kv_block; /* granularity of fwd_mask */
   int32_t bwd_query_block, bwd_kv_block; /* granularity of dq_mask (swapped) and dkdv_mask */
   int32_t dtype;                         /* KVAX_BF16 or KVAX_F16 */
-  int32_t flags;                         /* must be 0 */
+  int32_t flags;                         /* KVAX_FA_* bits */
   float scale;
   int32_t reserved;
 } kvax_fa_args;

@@ -12,6 +12,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libkvax_amd.so"
 ABI_VERSION = 1
 KVAX_MAX_MASKS = 4
 KVAX_BF16, KVAX_F16 = 0, 1
+KVAX_FA_DKDV_F32 = 1
 
 
 class KvaxNativeError(RuntimeError):

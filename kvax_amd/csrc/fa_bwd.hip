@@ -1,0 +1,643 @@
+// Flash-attention backward for gfx950: delta pre-pass, dQ kernel (query-stationary) and dK/dV
+// kernel (kv-stationary, all query heads of a GQA group reduced in registers).
+//
+// Semantics: reference kvax/ops/flash_attention_triton.py:373-410 (delta = rowsum(O * dO)),
+// :526-617 / :620-871 (dQ: P = exp2(S * scale * log2e - lse), dS = P * (dP - delta),
+// dQ = scale * dS K) and :413-523 / :874-1191 (dV = P^T dO, dK = scale * dS^T Q, summed over the
+// query heads of each kv head as :1855-1868 does).  P and dS are rounded to the input dtype
+// before the second contractions, as in the reference.  Padding tokens take part in nothing and
+// get exact-zero gradients.
+//
+// Layout trick shared with the forward: each contraction is arranged so that the tile produced
+// by the first MFMA stage (P or dS in C layout: one column per lane) is directly the B operand
+// of the second stage, whose A operand is gathered with transposing LDS reads.
+//   dQ kernel:    S^T, dP^T [kv x q]  ->  dQ^T [d x q]  += K^T [d x kv]  dS^T [kv x q]
+//   dK/dV kernel: S,   dP   [q x kv]  ->  dV^T [d x kv] += dO^T [d x q]  P  [q x kv]
+//                                         dK^T [d x kv] += Q^T  [d x q]  dS [q x kv]
+// Nothing is exchanged between wavefronts, no atomics are used and the result is deterministic.
+#include "common.h"
+#include "fa_common.h"
+
+namespace kvax {
+int validate_fa_common(const kvax_fa_args* a);
+
+namespace {
+
+constexpr int kTile = 64;  // rows of the streamed operand per LDS stage
+
+struct BwdParams {
+  const char* q;
+  const char* k;
+  const char* v;
+  const char* out;
+  const char* dout;
+  char* dq;
+  char* dk;
+  char* dv;
+  const float* lse;
+  float* delta;
+  const int32_t* q_pos;
+  const int32_t* q_seg;
+  const int32_t* kv_pos;
+  const int32_t* kv_seg;
+  const int32_t* dq_mask[4];
+  const int32_t* dkdv_mask[4];
+  int64_t q_sb, q_ss, q_sh;
+  int64_t k_sb, k_ss, k_sh;
+  int64_t v_sb, v_ss, v_sh;
+  int64_t o_sb, o_ss, o_sh;
+  int64_t do_sb, do_ss, do_sh;
+  int64_t dq_sb, dq_ss, dq_sh;
+  int64_t dk_sb, dk_ss, dk_sh;
+  int64_t dv_sb, dv_ss, dv_sh;
+  int batch, q_len, kv_len, num_heads, num_kv_heads, group;
+  int bq, bk;  // backward block sizes: the dQ mask has query blocks of bk and kv blocks of bq
+  int n_dq_blocks, n_kv_blocks;
+  int num_tiles, total_items;
+  int dkdv_f32;  // dK / dV are fp32 tensors (strides still in elements)
+  float scale, scale_log2;
+};
+
+// ---------------------------------------------------------------------------------------------
+// delta[b, h, i] = sum_d O[b, i, h, d] * dO[b, i, h, d]
+// ---------------------------------------------------------------------------------------------
+template <class Tr, int D>
+__global__ __launch_bounds__(256) void fa_bwd_delta_kernel(const BwdParams p) {
+  constexpr int kLanesPerRow = D / 8;
+  constexpr int kRowsPerGroup = 256 / kLanesPerRow;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerGroup + threadIdx.x / kLanesPerRow;
+  const int part = threadIdx.x % kLanesPerRow;
+  const int64_t total = (int64_t)p.batch * p.q_len * p.num_heads;
+  float acc = 0.f;
+  int b = 0, i = 0, hd = 0;
+  if (row < total) {
+    hd = (int)(row % p.num_heads);
+    i = (int)((row / p.num_heads) % p.q_len);
+    b = (int)(row / ((int64_t)p.num_heads * p.q_len));
+    const uint4 o = *reinterpret_cast<const uint4*>(
+        p.out + (b * p.o_sb + i * p.o_ss + hd * p.o_sh) * 2 + part * 16);
+    const uint4 g = *reinterpret_cast<const uint4*>(
+        p.dout + (b * p.do_sb + i * p.do_ss + hd * p.do_sh) * 2 + part * 16);
+    const uint32_t ow[4] = {o.x, o.y, o.z, o.w}, gw[4] = {g.x, g.y, g.z, g.w};
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      acc += Tr::to_float((uint16_t)(ow[w] & 0xffff)) * Tr::to_float((uint16_t)(gw[w] & 0xffff));
+      acc += Tr::to_float((uint16_t)(ow[w] >> 16)) * Tr::to_float((uint16_t)(gw[w] >> 16));
+    }
+  }
+#pragma unroll
+  for (int off = kLanesPerRow / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (row < total && part == 0) p.delta[((int64_t)b * p.num_heads + hd) * p.q_len + i] = acc;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Merged range of the streamed axis for a work-group that covers several mask blocks of the
+// stationary axis: union of [lower, upper), intersection of [lower_full, upper_full), in elements.
+// ---------------------------------------------------------------------------------------------
+struct Range {
+  int lo, hi, flo, fhi, min_hi, max_lo;
+};
+
+__device__ __forceinline__ Range merged_range(const int32_t* const mask[4], int64_t base, int blk0,
+                                              int blk1, int unit, int limit) {
+  Range r{0x7fffffff, 0, 0, 0x7fffffff, 0x7fffffff, 0};
+  for (int blk = blk0; blk <= blk1; blk++) {
+    const int l_ = mask[0][base + blk] * unit, u_ = mask[1][base + blk] * unit;
+    r.flo = max(r.flo, mask[2][base + blk] * unit);
+    r.fhi = min(r.fhi, mask[3][base + blk] * unit);
+    if (u_ > l_) {
+      r.lo = min(r.lo, l_);
+      r.hi = max(r.hi, u_);
+      r.min_hi = min(r.min_hi, u_);
+      r.max_lo = max(r.max_lo, l_);
+    } else {  // a block with nothing to do: every tile needs the per-column range test
+      r.min_hi = 0;
+      r.max_lo = 0x7fffffff;
+    }
+  }
+  r.hi = min(r.hi, limit);
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------------
+// dQ: one work-group = NW wavefronts x 32 query rows of one (batch, head); streams K/V tiles.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct DqSmem {
+  static constexpr int kStride = D * 2 + 16;
+  static constexpr int kTileBytes = kTile * kStride;
+  static constexpr int kStage = 2 * kTileBytes + 2 * kTile * 4;
+  static constexpr int kTotal = 2 * kStage;
+};
+
+template <class Tr, int D, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p) {
+  using vec8 = typename Tr::vec8;
+  using Smem = DqSmem<D>;
+  constexpr int NT = NW * 64;
+  constexpr int TQ = NW * 32;
+  constexpr int KSTEPS = D / 16;
+  constexpr int DT = D / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int c = lane % 32, h = lane / 32;
+
+  int item = xcd_contiguous(blockIdx.x, p.total_items);
+  const int g = item % p.group;
+  item /= p.group;
+  const int q_tile = p.num_tiles - 1 - item % p.num_tiles;
+  item /= p.num_tiles;
+  const int kv_head = item % p.num_kv_heads;
+  const int b = item / p.num_kv_heads;
+  const int head = kv_head * p.group + g;
+  const int q0 = q_tile * TQ;
+
+  const int32_t* kv_seg = p.kv_seg + (int64_t)b * p.kv_len;
+  const int32_t* kv_pos = p.kv_pos + (int64_t)b * p.kv_len;
+  const char* kbase = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh) * 2;
+  const char* vbase = p.v + ((int64_t)b * p.v_sb + (int64_t)kv_head * p.v_sh) * 2;
+
+  const int qbs = p.bk, kbs = p.bq;  // the dQ mask swaps the backward block sizes
+  const int64_t mbase = (int64_t)b * p.n_dq_blocks;
+  const Range r = merged_range(p.dq_mask, mbase, q0 / qbs,
+                               min((q0 + TQ - 1) / qbs, p.n_dq_blocks - 1), kbs, p.kv_len);
+  const int t_lo = r.lo / kTile;
+  const int t_hi = r.hi > r.lo ? (r.hi + kTile - 1) / kTile : t_lo;
+  const int tf_lo = (r.flo + kTile - 1) / kTile, tf_hi = r.fhi / kTile;
+
+  // per-lane query column
+  const int qrow = q0 + wave * 32 + c;
+  const bool in = qrow < p.q_len;
+  const int qseg = in ? p.q_seg[(int64_t)b * p.q_len + qrow] : -1;
+  const int qpos = in ? p.q_pos[(int64_t)b * p.q_len + qrow] : 0;
+  int col_lo = 0, col_hi = 0;
+  float lse_q = 0.f, delta_q = 0.f;
+  if (in && qseg != -1) {
+    col_lo = p.dq_mask[0][mbase + qrow / qbs] * kbs;
+    col_hi = p.dq_mask[1][mbase + qrow / qbs] * kbs;
+    lse_q = p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
+    delta_q = p.delta[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
+  }
+
+  f32x16 dq[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dq[dt][i] = 0.f;
+
+  if (t_hi > t_lo) {
+    vec8 qf[KSTEPS], dof[KSTEPS];
+    {
+      const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
+      const char* dr = p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh + (int64_t)(in ? qrow : 0) * p.do_ss) * 2;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        uint4 u = make_uint4(0, 0, 0, 0), w = make_uint4(0, 0, 0, 0);
+        if (in) {
+          u = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
+          w = *reinterpret_cast<const uint4*>(dr + (16 * ks + 8 * h) * 2);
+        }
+        qf[ks] = __builtin_bit_cast(vec8, u);
+        dof[ks] = __builtin_bit_cast(vec8, w);
+      }
+    }
+
+    RowTile<kTile, D, NT> kt_regs, vt_regs;
+    int32_t idreg = 0;
+    auto load_stage = [&](int kv0) {
+      kt_regs.load(kbase, p.k_ss * 2, kv0, p.kv_len, tid);
+      vt_regs.load(vbase, p.v_ss * 2, kv0, p.kv_len, tid);
+      if (tid < 2 * kTile) {
+        const int kv = kv0 + tid % kTile;
+        const bool is_seg = tid < kTile;
+        idreg = is_seg ? -1 : 0;
+        if (kv < p.kv_len) idreg = is_seg ? kv_seg[kv] : kv_pos[kv];
+      }
+    };
+    auto store_stage = [&](char* stage) {
+      kt_regs.store(stage, Smem::kStride, tid);
+      vt_regs.store(stage + Smem::kTileBytes, Smem::kStride, tid);
+      if (tid < 2 * kTile) reinterpret_cast<int32_t*>(stage + 2 * Smem::kTileBytes)[tid] = idreg;
+    };
+
+    load_stage(t_lo * kTile);
+    store_stage(smem);
+    __syncthreads();
+
+    for (int t = t_lo; t < t_hi; t++) {
+      const int kv0 = t * kTile;
+      char* stage = smem + ((t - t_lo) & 1) * Smem::kStage;
+      char* next_stage = smem + ((t - t_lo + 1) & 1) * Smem::kStage;
+      const bool has_next = t + 1 < t_hi;
+      if (has_next) load_stage(kv0 + kTile);
+      const char* ktile = stage;
+      const char* vtile = stage + Smem::kTileBytes;
+      const int32_t* ids = reinterpret_cast<const int32_t*>(stage + 2 * Smem::kTileBytes);
+      const bool full = t >= tf_lo && t < tf_hi;
+      const bool range_test = kv0 < r.max_lo || kv0 + kTile > r.min_hi;
+
+      vec8 dsb[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+          const vec8 ka = read_row8<Tr>(ktile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
+          const vec8 va = read_row8<Tr>(vtile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
+          s = Tr::mfma(ka, qf[ks], s);
+          dp = Tr::mfma(va, dof[ks], dp);
+        }
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const int r0 = 32 * kt + 8 * g4 + 4 * h;
+          int sg[4] = {0, 0, 0, 0}, ps[4] = {0, 0, 0, 0};
+          if (!full) {
+            const int4 ksg = *reinterpret_cast<const int4*>(ids + r0);
+            const int4 kps = *reinterpret_cast<const int4*>(ids + kTile + r0);
+            sg[0] = ksg.x, sg[1] = ksg.y, sg[2] = ksg.z, sg[3] = ksg.w;
+            ps[0] = kps.x, ps[1] = kps.y, ps[2] = kps.z, ps[3] = kps.w;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const int i = 4 * g4 + j;
+            float pr = fast_exp2(s[i] * p.scale_log2 - lse_q);
+            if (!full) {
+              bool ok = (sg[j] == qseg) && (qpos >= ps[j]);
+              if (range_test) {
+                const int kv = kv0 + r0 + j;
+                ok = ok && kv >= col_lo && kv < col_hi;
+              } else {
+                ok = ok && col_hi > 0;
+              }
+              if (!ok) pr = 0.f;
+            }
+            s[i] = pr * (dp[i] - delta_q);
+          }
+        }
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+          dsb[kt][st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                                  s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+      }
+      // dQ^T += K^T dS^T
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++) {
+            const vec8 a = tr_read_a<Tr>(ktile, Smem::kStride, 32 * kt + 16 * st, 32 * dt, lane);
+            dq[dt] = Tr::mfma(a, dsb[kt][st], dq[dt]);
+          }
+      if (has_next) store_stage(next_stage);
+      __syncthreads();
+    }
+  }
+
+  if (in) {
+    char* row = p.dq + ((int64_t)b * p.dq_sb + (int64_t)head * p.dq_sh + (int64_t)qrow * p.dq_ss) * 2;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        uint2 u;
+        u.x = Tr::pack2(dq[dt][4 * g4 + 0] * p.scale, dq[dt][4 * g4 + 1] * p.scale);
+        u.y = Tr::pack2(dq[dt][4 * g4 + 2] * p.scale, dq[dt][4 * g4 + 3] * p.scale);
+        *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dK/dV: one work-group = NW wavefronts x 32 kv rows of one (batch, kv head); streams the Q / dO
+// tiles of every query head of the group and accumulates dK^T, dV^T in registers.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct DkdvSmem {
+  static constexpr int kStride = D * 2 + 16;
+  static constexpr int kTileBytes = kTile * kStride;
+  static constexpr int kRowData = 4 * kTile * 4;  // lse, delta, seg, pos
+  static constexpr int kStage = 2 * kTileBytes + kRowData;
+  static constexpr int kTotal = 2 * kStage;
+};
+
+template <class Tr, int D, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams p) {
+  using vec8 = typename Tr::vec8;
+  using Smem = DkdvSmem<D>;
+  constexpr int NT = NW * 64;
+  constexpr int TKV = NW * 32;
+  constexpr int KSTEPS = D / 16;
+  constexpr int DT = D / 32;
+  static_assert(NT >= 4 * kTile, "row data is staged by one thread per value");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int c = lane % 32, h = lane / 32;
+
+  // early kv tiles see the most queries under a causal mask: run them first
+  int item = xcd_contiguous(blockIdx.x, p.total_items);
+  const int kv_tile = item % p.num_tiles;
+  item /= p.num_tiles;
+  const int kv_head = item % p.num_kv_heads;
+  const int b = item / p.num_kv_heads;
+  const int k0 = kv_tile * TKV;
+
+  const int kbs = p.bk, qbs = p.bq;
+  const int64_t mbase = (int64_t)b * p.n_kv_blocks;
+  const Range r = merged_range(p.dkdv_mask, mbase, k0 / kbs,
+                               min((k0 + TKV - 1) / kbs, p.n_kv_blocks - 1), qbs, p.q_len);
+  const int t_lo = r.lo / kTile;
+  const int t_hi = r.hi > r.lo ? (r.hi + kTile - 1) / kTile : t_lo;
+  const int tf_lo = (r.flo + kTile - 1) / kTile, tf_hi = r.fhi / kTile;
+  const int nt = t_hi - t_lo;
+
+  // per-lane kv column
+  const int kvcol = k0 + wave * 32 + c;
+  const bool in = kvcol < p.kv_len;
+  const int kvseg = in ? p.kv_seg[(int64_t)b * p.kv_len + kvcol] : -1;
+  const int kvpos = in ? p.kv_pos[(int64_t)b * p.kv_len + kvcol] : 0;
+  int col_lo = 0, col_hi = 0;
+  if (in && kvseg != -1) {
+    col_lo = p.dkdv_mask[0][mbase + kvcol / kbs] * qbs;
+    col_hi = p.dkdv_mask[1][mbase + kvcol / kbs] * qbs;
+  }
+
+  f32x16 dk[DT], dv[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) dk[dt][i] = 0.f, dv[dt][i] = 0.f;
+
+  if (nt > 0) {
+    vec8 kf[KSTEPS], vf[KSTEPS];
+    {
+      const char* kr = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh + (int64_t)(in ? kvcol : 0) * p.k_ss) * 2;
+      const char* vr = p.v + ((int64_t)b * p.v_sb + (int64_t)kv_head * p.v_sh + (int64_t)(in ? kvcol : 0) * p.v_ss) * 2;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        uint4 u = make_uint4(0, 0, 0, 0), w = make_uint4(0, 0, 0, 0);
+        if (in) {
+          u = *reinterpret_cast<const uint4*>(kr + (16 * ks + 8 * h) * 2);
+          w = *reinterpret_cast<const uint4*>(vr + (16 * ks + 8 * h) * 2);
+        }
+        kf[ks] = __builtin_bit_cast(vec8, u);
+        vf[ks] = __builtin_bit_cast(vec8, w);
+      }
+    }
+
+    RowTile<kTile, D, NT> q_regs, do_regs;
+    float rowreg = 0.f;
+    auto load_stage = [&](int step) {
+      const int head = kv_head * p.group + step / nt;
+      const int qr0 = (t_lo + step % nt) * kTile;
+      q_regs.load(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, p.q_ss * 2, qr0, p.q_len, tid);
+      do_regs.load(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, p.do_ss * 2, qr0, p.q_len, tid);
+      if (tid < 4 * kTile) {
+        const int which = tid / kTile;
+        const int qi = qr0 + tid % kTile;
+        const bool ok = qi < p.q_len;
+        const int64_t hoff = ((int64_t)b * p.num_heads + head) * p.q_len + qi;
+        const int64_t boff = (int64_t)b * p.q_len + qi;
+        if (which == 0) rowreg = ok ? p.lse[hoff] : 0.f;
+        else if (which == 1) rowreg = ok ? p.delta[hoff] : 0.f;
+        else if (which == 2) rowreg = __int_as_float(ok ? p.q_seg[boff] : -1);
+        else rowreg = __int_as_float(ok ? p.q_pos[boff] : 0);
+      }
+    };
+    auto store_stage = [&](char* stage) {
+      q_regs.store(stage, Smem::kStride, tid);
+      do_regs.store(stage + Smem::kTileBytes, Smem::kStride, tid);
+      if (tid < 4 * kTile) reinterpret_cast<float*>(stage + 2 * Smem::kTileBytes)[tid] = rowreg;
+    };
+
+    const int steps = nt * p.group;
+    load_stage(0);
+    store_stage(smem);
+    __syncthreads();
+
+    for (int step = 0; step < steps; step++) {
+      const int t = t_lo + step % nt;
+      const int qr0 = t * kTile;
+      char* stage = smem + (step & 1) * Smem::kStage;
+      char* next_stage = smem + ((step + 1) & 1) * Smem::kStage;
+      const bool has_next = step + 1 < steps;
+      if (has_next) load_stage(step + 1);
+      const char* qtile = stage;
+      const char* dotile = stage + Smem::kTileBytes;
+      const float* rowdata = reinterpret_cast<const float*>(stage + 2 * Smem::kTileBytes);
+      const bool full = t >= tf_lo && t < tf_hi;
+      const bool range_test = qr0 < r.max_lo || qr0 + kTile > r.min_hi;
+
+#pragma unroll
+      for (int mt = 0; mt < 2; mt++) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+          const vec8 qa = read_row8<Tr>(qtile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
+          const vec8 da = read_row8<Tr>(dotile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
+          s = Tr::mfma(qa, kf[ks], s);
+          dp = Tr::mfma(da, vf[ks], dp);
+        }
+        vec8 pb[2], dsb[2];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const int r0 = 32 * mt + 8 * g4 + 4 * h;
+          const float4 lse4 = *reinterpret_cast<const float4*>(rowdata + r0);
+          const float4 del4 = *reinterpret_cast<const float4*>(rowdata + kTile + r0);
+          const float ls[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
+          const float dl[4] = {del4.x, del4.y, del4.z, del4.w};
+          int sg[4] = {0, 0, 0, 0}, ps[4] = {0, 0, 0, 0};
+          if (!full) {
+            const int4 qsg = *reinterpret_cast<const int4*>(rowdata + 2 * kTile + r0);
+            const int4 qps = *reinterpret_cast<const int4*>(rowdata + 3 * kTile + r0);
+            sg[0] = qsg.x, sg[1] = qsg.y, sg[2] = qsg.z, sg[3] = qsg.w;
+            ps[0] = qps.x, ps[1] = qps.y, ps[2] = qps.z, ps[3] = qps.w;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const int i = 4 * g4 + j;
+            float pr = fast_exp2(s[i] * p.scale_log2 - ls[j]);
+            if (!full) {
+              bool ok = (sg[j] == kvseg) && (ps[j] >= kvpos);
+              if (range_test) {
+                const int qi = qr0 + r0 + j;
+                ok = ok && qi >= col_lo && qi < col_hi;
+              } else {
+                ok = ok && col_hi > 0;
+              }
+              if (!ok) pr = 0.f;
+            }
+            s[i] = pr;
+            dp[i] = pr * (dp[i] - dl[j]);
+          }
+        }
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+          pb[st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                             s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+          dsb[st] = pack8<Tr>(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
+                              dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
+        }
+        // dV^T += dO^T P ; dK^T += Q^T dS
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++) {
+            const vec8 ad = tr_read_a<Tr>(dotile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
+            dv[dt] = Tr::mfma(ad, pb[st], dv[dt]);
+            const vec8 aq = tr_read_a<Tr>(qtile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
+            dk[dt] = Tr::mfma(aq, dsb[st], dk[dt]);
+          }
+      }
+      if (has_next) store_stage(next_stage);
+      __syncthreads();
+    }
+  }
+
+  if (in && p.dkdv_f32) {
+    float* krow = reinterpret_cast<float*>(p.dk) + (int64_t)b * p.dk_sb + (int64_t)kv_head * p.dk_sh + (int64_t)kvcol * p.dk_ss;
+    float* vrow = reinterpret_cast<float*>(p.dv) + (int64_t)b * p.dv_sb + (int64_t)kv_head * p.dv_sh + (int64_t)kvcol * p.dv_ss;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const int d0 = 32 * dt + 8 * g4 + 4 * h;
+        *reinterpret_cast<float4*>(krow + d0) =
+            make_float4(dk[dt][4 * g4 + 0] * p.scale, dk[dt][4 * g4 + 1] * p.scale,
+                        dk[dt][4 * g4 + 2] * p.scale, dk[dt][4 * g4 + 3] * p.scale);
+        *reinterpret_cast<float4*>(vrow + d0) =
+            make_float4(dv[dt][4 * g4 + 0], dv[dt][4 * g4 + 1], dv[dt][4 * g4 + 2], dv[dt][4 * g4 + 3]);
+      }
+  } else if (in) {
+    char* krow = p.dk + ((int64_t)b * p.dk_sb + (int64_t)kv_head * p.dk_sh + (int64_t)kvcol * p.dk_ss) * 2;
+    char* vrow = p.dv + ((int64_t)b * p.dv_sb + (int64_t)kv_head * p.dv_sh + (int64_t)kvcol * p.dv_ss) * 2;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        uint2 u, w;
+        u.x = Tr::pack2(dk[dt][4 * g4 + 0] * p.scale, dk[dt][4 * g4 + 1] * p.scale);
+        u.y = Tr::pack2(dk[dt][4 * g4 + 2] * p.scale, dk[dt][4 * g4 + 3] * p.scale);
+        w.x = Tr::pack2(dv[dt][4 * g4 + 0], dv[dt][4 * g4 + 1]);
+        w.y = Tr::pack2(dv[dt][4 * g4 + 2], dv[dt][4 * g4 + 3]);
+        *reinterpret_cast<uint2*>(krow + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
+        *reinterpret_cast<uint2*>(vrow + (32 * dt + 8 * g4 + 4 * h) * 2) = w;
+      }
+  }
+}
+
+template <class K>
+int reserve_lds(K kernel, int bytes, bool* done, const char* what) {
+  if (*done) return KVAX_OK;
+  if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
+      hipSuccess)
+    return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for %s", bytes, what);
+  *done = true;
+  return KVAX_OK;
+}
+
+template <class Tr, int D>
+int launch_bwd(BwdParams p, hipStream_t stream) {
+  constexpr int NW = 4;
+  // delta
+  {
+    const int64_t rows = (int64_t)p.batch * p.q_len * p.num_heads;
+    constexpr int kRowsPerGroup = 256 / (D / 8);
+    if (rows > 0)
+      hipLaunchKernelGGL((fa_bwd_delta_kernel<Tr, D>), dim3((unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup)),
+                       dim3(256), 0, stream, p);
+    if (int rc = check_launch("fa_bwd_delta_kernel")) return rc;
+  }
+  // dQ
+  if (p.q_len > 0) {
+    auto kernel = fa_bwd_dq_kernel<Tr, D, NW>;
+    static bool done = false;
+    if (int rc = reserve_lds(kernel, DqSmem<D>::kTotal, &done, "the dQ kernel")) return rc;
+    p.num_tiles = cdiv(p.q_len, NW * 32);
+    p.total_items = p.batch * p.num_heads * p.num_tiles;
+    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), DqSmem<D>::kTotal, stream, p);
+    if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
+  }
+  // dK/dV
+  if (p.kv_len > 0) {
+    auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW>;
+    static bool done = false;
+    if (int rc = reserve_lds(kernel, DkdvSmem<D>::kTotal, &done, "the dK/dV kernel")) return rc;
+    p.num_tiles = cdiv(p.kv_len, NW * 32);
+    p.total_items = p.batch * p.num_kv_heads * p.num_tiles;
+    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), DkdvSmem<D>::kTotal, stream, p);
+    if (int rc = check_launch("fa_bwd_dkdv_kernel")) return rc;
+  }
+  return KVAX_OK;
+}
+
+}  // namespace
+}  // namespace kvax
+
+using namespace kvax;
+
+extern "C" size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* a) {
+  if (!a || a->batch < 0 || a->q_len < 0 || a->num_heads < 0) return 0;
+  return (size_t)a->batch * a->num_heads * a->q_len * sizeof(float);  // delta
+}
+
+extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
+                           kvax_stream_t stream_) {
+  if (int rc = validate_fa_common(a)) return rc;
+  if (!a->dout || !a->dq || !a->dk || !a->dv) return fail(KVAX_EINVAL, "null gradient pointer");
+  if (a->bwd_query_block <= 0 || a->bwd_kv_block <= 0)
+    return fail(KVAX_EINVAL, "backward block sizes must be positive");
+  for (int i = 0; i < 4; i++)
+    if (!a->dq_mask[i] || !a->dkdv_mask[i]) return fail(KVAX_EINVAL, "backward masks are missing");
+  const int64_t* strides[] = {a->do_strides, a->dq_strides, a->dk_strides, a->dv_strides};
+  for (auto s : strides)
+    for (int i = 0; i < 3; i++)
+      if (s[i] % 8) return fail(KVAX_EINVAL, "strides must be multiples of 8 elements (16 bytes)");
+  const void* ptrs[] = {a->dout, a->dq, a->dk, a->dv};
+  for (auto ptr : ptrs)
+    if ((uintptr_t)ptr % 16) return fail(KVAX_EINVAL, "tensor pointers must be 16-byte aligned");
+  const size_t need = kvax_fa_bwd_workspace_bytes(a);
+  if (need > workspace_bytes || (need && !workspace))
+    return fail(KVAX_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  if ((uintptr_t)workspace % 16) return fail(KVAX_EINVAL, "workspace must be 16-byte aligned");
+  if (a->batch == 0) return KVAX_OK;
+
+  BwdParams p{};
+  p.q = (const char*)a->q, p.k = (const char*)a->k, p.v = (const char*)a->v;
+  p.out = (const char*)a->out, p.dout = (const char*)a->dout;
+  p.dq = (char*)a->dq, p.dk = (char*)a->dk, p.dv = (char*)a->dv;
+  p.lse = a->lse;
+  p.delta = (float*)workspace;
+  p.q_pos = a->q_pos, p.q_seg = a->q_seg, p.kv_pos = a->kv_pos, p.kv_seg = a->kv_seg;
+  for (int i = 0; i < 4; i++) p.dq_mask[i] = a->dq_mask[i], p.dkdv_mask[i] = a->dkdv_mask[i];
+  p.q_sb = a->q_strides[0], p.q_ss = a->q_strides[1], p.q_sh = a->q_strides[2];
+  p.k_sb = a->k_strides[0], p.k_ss = a->k_strides[1], p.k_sh = a->k_strides[2];
+  p.v_sb = a->v_strides[0], p.v_ss = a->v_strides[1], p.v_sh = a->v_strides[2];
+  p.o_sb = a->o_strides[0], p.o_ss = a->o_strides[1], p.o_sh = a->o_strides[2];
+  p.do_sb = a->do_strides[0], p.do_ss = a->do_strides[1], p.do_sh = a->do_strides[2];
+  p.dq_sb = a->dq_strides[0], p.dq_ss = a->dq_strides[1], p.dq_sh = a->dq_strides[2];
+  p.dk_sb = a->dk_strides[0], p.dk_ss = a->dk_strides[1], p.dk_sh = a->dk_strides[2];
+  p.dv_sb = a->dv_strides[0], p.dv_ss = a->dv_strides[1], p.dv_sh = a->dv_strides[2];
+  p.batch = a->batch, p.q_len = a->q_len, p.kv_len = a->kv_len;
+  p.num_heads = a->num_heads, p.num_kv_heads = a->num_kv_heads;
+  p.group = a->num_heads / a->num_kv_heads;
+  p.bq = a->bwd_query_block, p.bk = a->bwd_kv_block;
+  p.n_dq_blocks = cdiv(a->q_len, a->bwd_kv_block);
+  p.n_kv_blocks = cdiv(a->kv_len, a->bwd_kv_block);
+  p.dkdv_f32 = (a->flags & KVAX_FA_DKDV_F32) != 0;
+  p.scale = a->scale;
+  p.scale_log2 = a->scale * 1.4426950408889634f;
+  hipStream_t stream = (hipStream_t)stream_;
+  const bool bf16 = a->dtype == KVAX_BF16;
+  if (a->head_dim == 128)
+    return bf16 ? launch_bwd<Bf16, 128>(p, stream) : launch_bwd<F16, 128>(p, stream);
+  return bf16 ? launch_bwd<Bf16, 64>(p, stream) : launch_bwd<F16, 64>(p, stream);
+}

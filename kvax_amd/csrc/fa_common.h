@@ -120,4 +120,36 @@ __device__ __forceinline__ int xcd_contiguous(int linear, int total) {
   return xcd * per + (xcd < rem ? xcd : rem) + idx;
 }
 
+
+// Cooperative staging of a ROWS x D tile of 16-bit elements: global -> registers (issued early
+// so the loads are in flight during compute) -> LDS rows of `lds_stride` bytes.  Rows at or
+// beyond `limit` are zero-filled.
+template <int ROWS, int D, int NT>
+struct RowTile {
+  static constexpr int kChunksPerRow = D / 8;  // 16-byte chunks
+  static constexpr int kPerThread = ROWS * kChunksPerRow / NT;
+  static_assert(ROWS * kChunksPerRow % NT == 0, "tile must split evenly over the work-group");
+  uint4 reg[kPerThread];
+
+  __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int row0,
+                                       int limit, int tid) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) {
+      const int id = tid + i * NT;
+      const int row = row0 + id / kChunksPerRow, ch = id % kChunksPerRow;
+      reg[i] = make_uint4(0, 0, 0, 0);
+      if (row < limit)
+        reg[i] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride_bytes + ch * 16);
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int lds_stride, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kPerThread; i++) {
+      const int id = tid + i * NT;
+      *reinterpret_cast<uint4*>(lds + (id / kChunksPerRow) * lds_stride + (id % kChunksPerRow) * 16) =
+          reg[i];
+    }
+  }
+};
+
 }  // namespace kvax

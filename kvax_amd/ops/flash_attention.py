@@ -118,11 +118,13 @@ def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd
 
 
 def flash_attention_backward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, dq_mask, dkdv_mask,
-                             out, lse, dout, scale, fwd_params, bwd_params):
-    """One device's backward: returns (dq, dk, dv) in the dtype of query."""
+                             out, lse, dout, scale, fwd_params, bwd_params, dkdv_fp32=False):
+    """One device's backward: returns (dq, dk, dv); dq in the dtype of query, dk / dv too unless
+    ``dkdv_fp32`` asks for the kernels' fp32 accumulators (used to sum context shards)."""
     dq = torch.empty_like(query)
-    dk = torch.empty_like(key)
-    dv = torch.empty_like(value)
+    kv_dtype = torch.float32 if dkdv_fp32 else key.dtype
+    dk = torch.empty(key.shape, dtype=kv_dtype, device=key.device)
+    dv = torch.empty(value.shape, dtype=kv_dtype, device=value.device)
     dout = dout if dout.stride(3) == 1 else dout.contiguous()
     a = _base_args(query, key, value, q_pos, q_seg, kv_pos, kv_seg, scale, fwd_params, bwd_params)
     a.out, a.lse, a.o_strides = out.data_ptr(), lse.data_ptr(), _strides3(out)
@@ -130,6 +132,7 @@ def flash_attention_backward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, dq
     a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     a.dq_strides, a.dk_strides, a.dv_strides = _strides3(dq), _strides3(dk), _strides3(dv)
     a.dq_mask, a.dkdv_mask = _mask_ptrs(dq_mask), _mask_ptrs(dkdv_mask)
+    a.flags = _native.KVAX_FA_DKDV_F32 if dkdv_fp32 else 0
     lib = _native.lib()
     if not hasattr(lib, "kvax_fa_bwd"):
         raise _native.KvaxNativeError("libkvax_amd.so was built without kvax_fa_bwd")
@@ -202,10 +205,10 @@ class _FlashAttentionFn(torch.autograd.Function):
                 query[:, sl], key, value, q_pos[:, sl].contiguous(), q_seg[:, sl].contiguous(),
                 kv_pos, kv_seg, _slice_mask(masks[1], r, cp, False),
                 _slice_mask(masks[2], r, cp, True), out[:, sl], lse[:, :, sl].contiguous(),
-                dout[:, sl], ctx.scale, ctx.fwd_params, bwd)
+                dout[:, sl], ctx.scale, ctx.fwd_params, bwd, dkdv_fp32=cp > 1)
             dqs.append(dq_r)
             if dk is None:
-                dk, dv = (dk_r.float(), dv_r.float()) if cp > 1 else (dk_r, dv_r)
+                dk, dv = dk_r, dv_r
             else:
                 dk += dk_r
                 dv += dv_r

@@ -1,0 +1,187 @@
+"""Backward parity of the HIP flash-attention kernels (through the C ABI and the autograd
+wrapper) with the dense CPU oracle.
+
+Tolerance: max abs error <= 2e-2 on dQ, dK, dV (the build's target).  Two refinements where the
+number format, not the kernel, sets the floor: (1) for |gradient| >= 2 a bf16 result rounds by up
+to 7.8e-3..3.1e-2, so the reference's relative bound is added above 2 (rtol 1e-2 for dQ, 3e-2 for
+dK/dV, kvax/utils/benchmarking.py:614-627); (2) dK/dV are additionally checked as fp32 (the
+reference kernels' own output type) against the plain 2e-2 bound in
+``test_fp32_dkdv_within_plain_bound``.
+"""
+import numpy as np
+import pytest
+import torch
+
+from kvax_amd import create_attention_mask, flash_attention
+from kvax_amd.utils import FlashAttentionParamsConfig, attention_specs
+from kvax_amd.utils.benchmarking import (
+    generate_random_segments_lengths,
+    make_random_attention_inputs,
+    workload,
+)
+from oracle import attention_oracle as ao
+
+pytestmark = pytest.mark.gpu
+TP_SPECS = (("data", None, "model", None), ("data", None, "model", None))
+ATOL = 2e-2
+
+
+def run_backward(data, scale, fwd_blocks, bwd_blocks, dout):
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    q, k, v = (x.detach().clone().requires_grad_(True) for x in (q, k, v))
+    fwd = FlashAttentionParamsConfig(*fwd_blocks)
+    bwd = FlashAttentionParamsConfig(*bwd_blocks)
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg, fwd_params=fwd, bwd_params=bwd,
+                                     calc_bwd_mask=True)
+        out = flash_attention(q, k, v, q_pos, q_seg, kv_pos, kv_seg, mask, scale=scale,
+                              fwd_params=fwd, bwd_params=bwd)
+    out.backward(dout)
+    return out.detach(), q.grad, k.grad, v.grad
+
+
+def oracle_backward(data, scale, dout, heads=None, dtype=np.float64, row_block=4096):
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = [x.cpu() for x in data]
+    return ao.attention_backward(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                 q_pos.numpy(), q_seg.numpy(), kv_pos.numpy(), kv_seg.numpy(),
+                                 scale, dout.float().cpu().numpy(), dtype=dtype, heads=heads,
+                                 row_block=row_block)
+
+
+def check_grad(name, got, ref, rtol, atol=ATOL):
+    got = got.float().cpu().numpy()
+    assert np.isfinite(got).all(), name
+    err = np.abs(got - ref)
+    bound = atol + rtol * np.maximum(np.abs(ref) - 2.0, 0.0)
+    worst = (err - bound).max()
+    assert worst <= 0, f"{name}: max abs err {err.max():.4g} (|ref| max {np.abs(ref).max():.3g})"
+    return err.max()
+
+
+def check_all(grads, refs, q_seg, kv_seg, kv_atol=ATOL):
+    dq, dk, dv = grads
+    check_grad("dq", dq, refs[0], 1e-2)
+    check_grad("dk", dk, refs[1], 3e-2, kv_atol)
+    check_grad("dv", dv, refs[2], 3e-2, kv_atol)
+    qpad = q_seg.cpu().numpy() == -1
+    kpad = kv_seg.cpu().numpy() == -1
+    assert (dq.float().cpu().numpy()[qpad] == 0).all(), "padding rows of dQ must be zero"
+    assert (dk.float().cpu().numpy()[kpad] == 0).all(), "padding rows of dK must be zero"
+    assert (dv.float().cpu().numpy()[kpad] == 0).all(), "padding rows of dV must be zero"
+
+
+# (q_len, kv_len, heads, kv_heads, head_dim, pad, segments, fwd blocks, bwd blocks): the shape
+# families of tests/test_attention.py:379-398 plus documents, GQA/MQA and mixed block sizes
+CASES = [
+    (384, 384, 8, 8, 64, 0, 1, (64, 64), (64, 64)),
+    (384, 384, 8, 8, 128, 0, 1, (64, 64), (64, 64)),
+    (256, 256, 8, 8, 128, 0, 1, (128, 128), (64, 128)),
+    (256, 256, 8, 8, 128, 200, 1, (64, 64), (64, 64)),
+    (256, 256, 16, 8, 128, 0, 1, (64, 64), (64, 64)),
+    (256, 256, 16, 1, 128, 0, 1, (64, 64), (128, 64)),
+    (1024, 1024, 8, 2, 128, 77, 5, (128, 128), (128, 128)),
+    (1024, 1024, 8, 2, 64, 0, 12, (64, 64), (64, 128)),
+    (2048, 2048, 4, 4, 128, 300, 7, (128, 128), (128, 128)),
+    (512, 1024, 4, 2, 128, 0, 1, (128, 128), (128, 128)),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_backward_matches_dense_oracle(device, case):
+    sq, sk, hq, hkv, d, pad, nseg, fwd_blocks, bwd_blocks = case
+    lengths = generate_random_segments_lengths(min(sq, sk), nseg)
+    start = sk - sq if sk > sq else 0
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d, d, seed=sq + d + hq,
+                                               num_pad_tokens=pad, start_query_position=start,
+                                               list_of_segment_lengths=lengths, device=device)
+    dout = torch.randn(data[0].shape, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(device)
+    _, dq, dk, dv = run_backward(data, scale, fwd_blocks, bwd_blocks, dout)
+    refs = oracle_backward(data, scale, dout)
+    # one kv head summing 16 query heads: the reference relaxes its bound to 5e-2 for this
+    # shape too (tests/test_attention.py:446-452)
+    check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if hkv == 1 else ATOL)
+
+
+@pytest.mark.parametrize("case", [CASES[7], CASES[6], CASES[8]])
+def test_fp32_dkdv_within_plain_bound(device, case):
+    """dK/dV straight from the fp32 accumulators: plain max abs error <= 2e-2, no relative term."""
+    from kvax_amd.ops.flash_attention import flash_attention_backward, flash_attention_forward
+
+    sq, sk, hq, hkv, d, pad, nseg, fwd_blocks, bwd_blocks = case
+    lengths = generate_random_segments_lengths(min(sq, sk), nseg)
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d, d, seed=sq + d + hq,
+                                               num_pad_tokens=pad,
+                                               list_of_segment_lengths=lengths, device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(device)
+    fwd, bwd = FlashAttentionParamsConfig(*fwd_blocks), FlashAttentionParamsConfig(*bwd_blocks)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg, fwd_params=fwd, bwd_params=bwd,
+                                      calc_bwd_mask=True)
+    out, lse = flash_attention_forward(q, k, v, q_pos, q_seg, kv_pos, kv_seg, masks[0], scale, fwd, bwd)
+    dq, dk, dv = flash_attention_backward(q, k, v, q_pos, q_seg, kv_pos, kv_seg, masks[1], masks[2],
+                                          out, lse, dout, scale, fwd, bwd, dkdv_fp32=True)
+    assert dk.dtype == torch.float32 and dv.dtype == torch.float32
+    refs = oracle_backward(data, scale, dout)
+    for name, got, ref in (("dk", dk, refs[1]), ("dv", dv, refs[2])):
+        err = np.abs(got.cpu().numpy() - ref).max()
+        assert err <= ATOL, f"{name}: max abs err {err:.4g}"
+
+
+def test_backward_fp16(device):
+    data, scale = make_random_attention_inputs(1, 512, 512, 4, 2, 128, 128, seed=3,
+                                               num_pad_tokens=50, dtype=torch.float16, device=device)
+    dout = torch.randn(data[0].shape, generator=torch.Generator().manual_seed(2)).to(torch.float16).to(device)
+    _, dq, dk, dv = run_backward(data, scale, (128, 128), (128, 128), dout)
+    check_all((dq, dk, dv), oracle_backward(data, scale, dout), data[4], data[6])
+
+
+def test_positions_restart_per_document(device):
+    w = workload("cpu_plumbing")
+    w.dtype = torch.bfloat16
+    q, k, v, dout = w.draw_tensors(0, device, with_dout=True)
+    data = (q, k, v) + w.ids(device)
+    _, dq, dk, dv = run_backward(data, w.scale, (64, 64), (64, 64), dout)
+    check_all((dq, dk, dv), oracle_backward(data, w.scale, dout), data[4], data[6])
+
+
+def test_gqa_equals_repeated_kv_heads(device):
+    data, scale = make_random_attention_inputs(1, 256, 256, 8, 2, 128, 128, seed=9, device=device)
+    q, k, v, *ids = data
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).to(device)
+    _, dq, dk, dv = run_backward(data, scale, (64, 64), (64, 64), dout)
+    k_rep, v_rep = k.repeat_interleave(4, dim=2), v.repeat_interleave(4, dim=2)
+    _, dq2, dk2, dv2 = run_backward((q, k_rep, v_rep, *ids), scale, (64, 64), (64, 64), dout)
+    assert (dq.float() - dq2.float()).abs().max().item() <= 1.6e-2
+    dk2 = dk2.float().reshape(1, 256, 2, 4, 128).sum(3)
+    dv2 = dv2.float().reshape(1, 256, 2, 4, 128).sum(3)
+    assert (dk.float() - dk2).abs().max().item() <= 3e-2
+    assert (dv.float() - dv2).abs().max().item() <= 3e-2
+
+
+@pytest.mark.parametrize("name, heads", [("doc32k", [8, 9, 10, 11]), ("block_skip", [56, 57, 58, 59, 60, 61, 62, 63])])
+def test_measurement_workloads_sampled_group(device, name, heads):
+    """Full-size configurations.  The oracle evaluates one whole GQA group so that dK/dV of its kv
+    head are complete; dQ is checked on those heads."""
+    w = workload(name)
+    q, k, v, dout = w.draw_tensors(0, device, with_dout=True)
+    data = (q, k, v) + w.ids(device)
+    _, dq, dk, dv = run_backward(data, w.scale, w.fwd_blocks, w.bwd_blocks, dout)
+    b = slice(0, 1)
+    refs = oracle_backward(tuple(x[b] for x in data), w.scale, dout[b], heads=heads,
+                           dtype=np.float32, row_block=2048)
+    kvh = heads[0] // (w.num_heads // w.num_kv_heads)
+    check_grad("dq", dq[b][:, :, heads], refs[0][:, :, heads], 1e-2)
+    check_grad("dk", dk[b][:, :, kvh], refs[1][:, :, kvh], 3e-2)
+    check_grad("dv", dv[b][:, :, kvh], refs[2][:, :, kvh], 3e-2)
+
+
+def test_missing_backward_masks(device):
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 64, 64, device=device)
+    q, k, v, *ids = data
+    q = q.clone().requires_grad_(True)
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(*ids)
+        out = flash_attention(q, k, v, *ids, mask, scale=scale)
+        with pytest.raises(ValueError):
+            out.sum().backward()
