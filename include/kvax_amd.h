@@ -85,8 +85,14 @@ int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const int32_t* k
  * :1421-1451) needs no kernel support: the caller passes those indices as q_pos / kv_pos.
  * ------------------------------------------------------------------------------------------ */
 enum {
-  KVAX_FA_DKDV_F32 = 1 /* backward writes dk / dv as fp32 (the reference kernels' output type,
-                          flash_attention_triton.py:1729-1730) instead of the dtype of q */
+  KVAX_FA_DKDV_F32 = 1,  /* backward writes dk / dv as fp32 (the reference kernels' output type,
+                            flash_attention_triton.py:1729-1730) instead of the dtype of q */
+  /* Backward phase selection, for profiling one kernel at a time.  The phases are the three
+   * launches of the reference's context-parallel path (:1692, :1740, :1778); skipping a phase
+   * leaves its outputs untouched (a skipped delta phase reuses the workspace contents). */
+  KVAX_FA_SKIP_DELTA = 16,
+  KVAX_FA_SKIP_DQ = 32,
+  KVAX_FA_SKIP_DKDV = 64
 };
 
 typedef struct kvax_fa_args {

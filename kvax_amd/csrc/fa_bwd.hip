@@ -55,6 +55,7 @@ struct BwdParams {
   int n_dq_blocks, n_kv_blocks;
   int num_tiles, total_items;
   int dkdv_f32;  // dK / dV are fp32 tensors (strides still in elements)
+  int flags;
   float scale, scale_log2;
 };
 
@@ -548,7 +549,7 @@ template <class Tr, int D>
 int launch_bwd(BwdParams p, hipStream_t stream) {
   constexpr int NW = 4;
   // delta
-  {
+  if (!(p.flags & KVAX_FA_SKIP_DELTA)) {
     const int64_t rows = (int64_t)p.batch * p.q_len * p.num_heads;
     constexpr int kRowsPerGroup = 256 / (D / 8);
     if (rows > 0)
@@ -557,7 +558,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     if (int rc = check_launch("fa_bwd_delta_kernel")) return rc;
   }
   // dQ
-  if (p.q_len > 0) {
+  if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
     auto kernel = fa_bwd_dq_kernel<Tr, D, NW>;
     static bool done = false;
     if (int rc = reserve_lds(kernel, DqSmem<D>::kTotal, &done, "the dQ kernel")) return rc;
@@ -567,7 +568,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
   }
   // dK/dV
-  if (p.kv_len > 0) {
+  if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
     auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW>;
     static bool done = false;
     if (int rc = reserve_lds(kernel, DkdvSmem<D>::kTotal, &done, "the dK/dV kernel")) return rc;
@@ -633,6 +634,7 @@ extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.n_dq_blocks = cdiv(a->q_len, a->bwd_kv_block);
   p.n_kv_blocks = cdiv(a->kv_len, a->bwd_kv_block);
   p.dkdv_f32 = (a->flags & KVAX_FA_DKDV_F32) != 0;
+  p.flags = a->flags;
   p.scale = a->scale;
   p.scale_log2 = a->scale * 1.4426950408889634f;
   hipStream_t stream = (hipStream_t)stream_;

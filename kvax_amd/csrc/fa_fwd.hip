@@ -395,7 +395,7 @@ int validate_fa_common(const kvax_fa_args* a) {
     return fail(KVAX_EUNSUPPORTED, "head_dim %d is not built (64 and 128 are)", a->head_dim);
   if (a->dtype != KVAX_BF16 && a->dtype != KVAX_F16)
     return fail(KVAX_EUNSUPPORTED, "dtype %d is not supported (bf16 and f16 are)", a->dtype);
-  if (a->flags & ~KVAX_FA_DKDV_F32) return fail(KVAX_EINVAL, "unknown bits in flags");
+  if (a->flags & ~(KVAX_FA_DKDV_F32 | KVAX_FA_SKIP_DELTA | KVAX_FA_SKIP_DQ | KVAX_FA_SKIP_DKDV)) return fail(KVAX_EINVAL, "unknown bits in flags");
   if (!a->q || !a->k || !a->v || !a->out || !a->lse || !a->q_pos || !a->q_seg || !a->kv_pos ||
       !a->kv_seg)
     return fail(KVAX_EINVAL, "null tensor pointer");

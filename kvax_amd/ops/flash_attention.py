@@ -100,11 +100,15 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
 
 
 def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd_mask, scale,
-                            fwd_params, bwd_params):
-    """One device's forward: returns (out like query, lse fp32 [batch, heads, q_len])."""
+                            fwd_params, bwd_params, buffers=None):
+    """One device's forward: returns (out like query, lse fp32 [batch, heads, q_len]).
+    ``buffers`` = (out, lse) lets a caller reuse its output tensors."""
     b, sq, hq, d = query.shape
-    out = torch.empty_like(query)
-    lse = torch.empty((b, hq, sq), dtype=torch.float32, device=query.device)
+    if buffers is not None:
+        out, lse = buffers
+    else:
+        out = torch.empty_like(query)
+        lse = torch.empty((b, hq, sq), dtype=torch.float32, device=query.device)
     a = _base_args(query, key, value, q_pos, q_seg, kv_pos, kv_seg, scale, fwd_params, bwd_params)
     a.out, a.lse, a.o_strides = out.data_ptr(), lse.data_ptr(), _strides3(out)
     a.fwd_mask = _mask_ptrs(fwd_mask)
@@ -118,13 +122,18 @@ def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd
 
 
 def flash_attention_backward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, dq_mask, dkdv_mask,
-                             out, lse, dout, scale, fwd_params, bwd_params, dkdv_fp32=False):
+                             out, lse, dout, scale, fwd_params, bwd_params, dkdv_fp32=False,
+                             flags=0, buffers=None):
     """One device's backward: returns (dq, dk, dv); dq in the dtype of query, dk / dv too unless
     ``dkdv_fp32`` asks for the kernels' fp32 accumulators (used to sum context shards)."""
-    dq = torch.empty_like(query)
     kv_dtype = torch.float32 if dkdv_fp32 else key.dtype
-    dk = torch.empty(key.shape, dtype=kv_dtype, device=key.device)
-    dv = torch.empty(value.shape, dtype=kv_dtype, device=value.device)
+    if buffers is not None:  # (dq, dk, dv, workspace) reused across calls, e.g. by the benchmark
+        dq, dk, dv, ws = buffers
+    else:
+        dq = torch.empty_like(query)
+        dk = torch.empty(key.shape, dtype=kv_dtype, device=key.device)
+        dv = torch.empty(value.shape, dtype=kv_dtype, device=value.device)
+        ws = None
     dout = dout if dout.stride(3) == 1 else dout.contiguous()
     a = _base_args(query, key, value, q_pos, q_seg, kv_pos, kv_seg, scale, fwd_params, bwd_params)
     a.out, a.lse, a.o_strides = out.data_ptr(), lse.data_ptr(), _strides3(out)
@@ -132,11 +141,12 @@ def flash_attention_backward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, dq
     a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     a.dq_strides, a.dk_strides, a.dv_strides = _strides3(dq), _strides3(dk), _strides3(dv)
     a.dq_mask, a.dkdv_mask = _mask_ptrs(dq_mask), _mask_ptrs(dkdv_mask)
-    a.flags = _native.KVAX_FA_DKDV_F32 if dkdv_fp32 else 0
+    a.flags = (_native.KVAX_FA_DKDV_F32 if dkdv_fp32 else 0) | flags
     lib = _native.lib()
     if not hasattr(lib, "kvax_fa_bwd"):
         raise _native.KvaxNativeError("libkvax_amd.so was built without kvax_fa_bwd")
-    ws = _workspace(lib.kvax_fa_bwd_workspace_bytes(C.byref(a)), query.device)
+    if ws is None:
+        ws = _workspace(lib.kvax_fa_bwd_workspace_bytes(C.byref(a)), query.device)
     with torch.cuda.device(query.device):
         stream = torch.cuda.current_stream().cuda_stream
         rc = lib.kvax_fa_bwd(C.byref(a), ws.data_ptr(), ws.numel(), C.c_void_p(stream))
