@@ -1,0 +1,135 @@
+"""Host-side logic and the C-ABI surface (no GPU): utils mirror the reference's behaviour, the
+shared library loads and exports every symbol the header declares, and the ops refuse to run
+without a GPU instead of falling back."""
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+import kvax_amd
+from kvax_amd import _native
+from kvax_amd.utils import (
+    PADDING_SEGMENT_ID,
+    FlashAttentionParamsConfig,
+    Mesh,
+    attention_specs,
+    permute_tokens_context_parallelism,
+    unpermute_tokens_context_parallelism,
+)
+from kvax_amd.utils.common import get_default_flash_attention_params, pad_to_block_size
+from kvax_amd.utils.math import get_multi_head_attention_tflops
+from kvax_amd.utils.permutation import generate_shard_indices
+from kvax_amd.utils.specs import get_attention_specs
+
+ROOT = Path(__file__).resolve().parent.parent
+CP = (("data", "context", None, None), ("data", None, None, None))
+
+
+def test_header_symbols_are_exported():
+    header = (ROOT / "include" / "kvax_amd.h").read_text()
+    declared = set(re.findall(r"\b(kvax_[a-z_0-9]+)\s*\(", header))
+    declared -= {"kvax_mask_desc", "kvax_fa_args"}
+    assert {"kvax_mask_build", "kvax_fa_fwd", "kvax_fa_bwd", "kvax_last_error"} <= declared
+    lib = _native.lib()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert lib.kvax_abi_version() == _native.ABI_VERSION
+
+
+def test_ctypes_structs_match_the_header_layout():
+    # 13 pointers + 12 mask pointers + 24 int64 strides + 14 int32/float fields
+    assert ctypes.sizeof(_native.FaArgs) == 13 * 8 + 12 * 8 + 24 * 8 + 14 * 4
+    assert ctypes.sizeof(_native.MaskDesc) == 4 * 4 + 4 * 8
+
+
+def test_argument_validation_without_a_gpu():
+    lib = _native.lib()
+    assert lib.kvax_fa_fwd(None, None, 0, None) == -1
+    assert b"null" in lib.kvax_last_error()
+    a = _native.FaArgs()
+    a.num_heads, a.num_kv_heads, a.head_dim = 8, 3, 128
+    assert lib.kvax_fa_fwd(ctypes.byref(a), None, 0, None) == -1
+    a.num_kv_heads, a.head_dim = 4, 48
+    assert lib.kvax_fa_fwd(ctypes.byref(a), None, 0, None) == -2
+    assert b"head_dim" in lib.kvax_last_error()
+    d = (_native.MaskDesc * 1)()
+    assert lib.kvax_mask_build(None, None, None, None, 1, 8, 8, 1, 1, d, 1, None, 0, None) == -1
+
+
+def test_ops_refuse_cpu_tensors():
+    ids = [torch.zeros((1, 64), dtype=torch.int32)] * 4
+    with attention_specs(("data", None, "model", None), ("data", None, "model", None)):
+        with pytest.raises(_native.KvaxNativeError):
+            kvax_amd.create_attention_mask(*ids)
+        q = torch.zeros((1, 64, 2, 64), dtype=torch.bfloat16)
+        with pytest.raises(_native.KvaxNativeError):
+            kvax_amd.flash_attention(q, q, q, *ids, mask=(None,))
+
+
+def test_public_surface():
+    for name in ("flash_attention", "create_attention_mask", "attention_specs", "PADDING_SEGMENT_ID",
+                 "FlashAttentionParamsConfig", "permute_tokens_context_parallelism",
+                 "unpermute_tokens_context_parallelism"):
+        assert name in kvax_amd.__all__ and hasattr(kvax_amd, name)
+    assert PADDING_SEGMENT_ID == -1
+    assert FlashAttentionParamsConfig() == FlashAttentionParamsConfig(64, 64, 4, 3)
+    assert get_default_flash_attention_params(backward=True).kv_block_size == 128
+
+
+def test_specs_validation_and_restore():
+    with pytest.raises(ValueError):
+        get_attention_specs()
+    with pytest.raises(ValueError, match="exactly 4"):
+        with attention_specs(("a", None, None), ("a", None, None, None)):
+            pass
+    with pytest.raises(ValueError, match="Batch"):
+        with attention_specs(("a", None, None, None), ("b", None, None, None)):
+            pass
+    with pytest.raises(ValueError, match="sharded key/value"):
+        with attention_specs(("a", "c", None, None), ("a", "c", None, None)):
+            pass
+    with pytest.raises(ValueError, match="head_dim"):
+        with attention_specs(("a", None, None, "x"), ("a", None, None, "x")):
+            pass
+    with attention_specs(*CP):
+        assert get_attention_specs().query_specs[1] == "context"
+        with attention_specs(("d", None, "m", None), ("d", None, "m", None)):
+            assert get_attention_specs().query_specs[1] is None
+        assert get_attention_specs().query_specs[1] == "context"
+    with pytest.raises(ValueError):
+        get_attention_specs()
+
+
+def test_permutation_closed_form_and_round_trip():
+    assert generate_shard_indices(8) == [0, 7, 1, 6, 2, 5, 3, 4]
+    x = torch.arange(2 * 64 * 3).reshape(2, 64, 3)
+    ids = torch.arange(64).expand(2, 64)
+    with attention_specs(*CP), Mesh({"data": 1, "context": 4, "model": 1}) as mesh:
+        px, pids = permute_tokens_context_parallelism((x, ids))
+        chunks = pids[0].reshape(8, 8)[:, 0] // 8
+        assert chunks.tolist() == [0, 7, 1, 6, 2, 5, 3, 4]
+        # shard r of 4 owns original chunks r and 7 - r
+        for r in range(4):
+            own = pids[0].reshape(4, 16)[r]
+            assert set((own // 8).tolist()) == {r, 7 - r}
+        back = unpermute_tokens_context_parallelism(px, mesh=mesh)
+        assert torch.equal(back, x)
+        assert torch.equal(unpermute_tokens_context_parallelism((pids,))[0], ids)
+    with attention_specs(*CP):
+        with pytest.raises(ValueError):
+            permute_tokens_context_parallelism(x)  # no mesh anywhere
+
+
+def test_pad_to_block_size_and_flops_model():
+    pos = torch.arange(10).reshape(1, 10)
+    seg = torch.zeros((1, 10), dtype=torch.int64)
+    emb = torch.ones((1, 10, 2, 4))
+    (e,), p, s = pad_to_block_size((emb,), pos, seg, 8, pos_fill_value=-7)
+    assert e.shape == (1, 16, 2, 4) and e[:, 10:].abs().sum() == 0
+    assert p[0, 10:].tolist() == [-7] * 6 and s[0, 10:].tolist() == [-1] * 6
+    t = get_multi_head_attention_tflops(2, 1024, 1024, 8, 128, 128, causal=True,
+                                        forward_pass=True, backward_pass=True)
+    assert t == pytest.approx(2 * 8 * 4 * 128 * 1024 * 1024 * 0.5 * 3.5 / 1e12)
