@@ -6,9 +6,10 @@ telling the caller to build it (``python -m kvax_amd.csrc.build``).
 from __future__ import annotations
 
 import ctypes as C
+import os
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "libkvax_amd.so"
+LIB_PATH = Path(os.environ.get("KVAX_AMD_LIB") or Path(__file__).resolve().parent / "libkvax_amd.so")
 ABI_VERSION = 1
 KVAX_MAX_MASKS = 4
 KVAX_BF16, KVAX_F16 = 0, 1

@@ -17,7 +17,7 @@ ROOT = PKG.parent
 LIB = PKG / "libkvax_amd.so"
 OBJ = CSRC / "build"
 
-SOURCES = ["abi.cpp", "mask_builder.hip", "fa_fwd.hip", "fa_bwd.hip"]
+SOURCES = ["abi.cpp", "mask_builder.hip", "fa_tiles.hip", "fa_fwd.hip", "fa_bwd.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -42,7 +42,13 @@ def _compile(src: str, extra: list[str]) -> Path:
     return out
 
 
-def build(extra_flags: list[str] | None = None, jobs: int = 4) -> Path:
+def build(extra_flags: list[str] | None = None, jobs: int = 4, lib: Path | None = None) -> Path:
+    """Compile and link; ``lib`` overrides the output path (used for experimental variants,
+    loaded by pointing the KVAX_AMD_LIB environment variable at them)."""
+    global LIB, OBJ
+    if lib is not None:
+        LIB = Path(lib).resolve()
+        OBJ = LIB.parent / (LIB.stem + "_obj")
     extra = list(extra_flags or [])
     sources = [s for s in SOURCES if (CSRC / s).exists()]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -55,4 +61,8 @@ def build(extra_flags: list[str] | None = None, jobs: int = 4) -> Path:
 
 
 if __name__ == "__main__":
-    print(build(sys.argv[1:]))
+    args = sys.argv[1:]
+    out = None
+    if args and args[0] == "-o":
+        out, args = Path(args[1]), args[2:]
+    print(build(args, lib=out))

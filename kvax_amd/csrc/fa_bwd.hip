@@ -23,7 +23,7 @@ int validate_fa_common(const kvax_fa_args* a);
 
 namespace {
 
-constexpr int kTile = 64;  // rows of the streamed operand per LDS stage
+constexpr int kTile = kTileRows;  // rows of the streamed operand per LDS stage
 
 struct BwdParams {
   const char* q;
@@ -55,6 +55,9 @@ struct BwdParams {
   int n_dq_blocks, n_kv_blocks;
   int num_tiles, total_items;
   int dkdv_f32;  // dK / dV are fp32 tensors (strides still in elements)
+  const int4* kv_tiles;  // tile summaries [batch, n_kv_tiles, 2]
+  const int4* q_tiles;   // tile summaries [batch, n_q_tiles, 2]
+  int n_kv_tiles, n_q_tiles;
   int flags;
   float scale, scale_log2;
 };
@@ -96,12 +99,12 @@ __global__ __launch_bounds__(256) void fa_bwd_delta_kernel(const BwdParams p) {
 // stationary axis: union of [lower, upper), intersection of [lower_full, upper_full), in elements.
 // ---------------------------------------------------------------------------------------------
 struct Range {
-  int lo, hi, flo, fhi, min_hi, max_lo;
+  int lo, hi, flo, fhi;
 };
 
 __device__ __forceinline__ Range merged_range(const int32_t* const mask[4], int64_t base, int blk0,
                                               int blk1, int unit, int limit) {
-  Range r{0x7fffffff, 0, 0, 0x7fffffff, 0x7fffffff, 0};
+  Range r{0x7fffffff, 0, 0, 0x7fffffff};
   for (int blk = blk0; blk <= blk1; blk++) {
     const int l_ = mask[0][base + blk] * unit, u_ = mask[1][base + blk] * unit;
     r.flo = max(r.flo, mask[2][base + blk] * unit);
@@ -109,11 +112,6 @@ __device__ __forceinline__ Range merged_range(const int32_t* const mask[4], int6
     if (u_ > l_) {
       r.lo = min(r.lo, l_);
       r.hi = max(r.hi, u_);
-      r.min_hi = min(r.min_hi, u_);
-      r.max_lo = max(r.max_lo, l_);
-    } else {  // a block with nothing to do: every tile needs the per-column range test
-      r.min_hi = 0;
-      r.max_lo = 0x7fffffff;
     }
   }
   r.hi = min(r.hi, limit);
@@ -173,14 +171,27 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
   const bool in = qrow < p.q_len;
   const int qseg = in ? p.q_seg[(int64_t)b * p.q_len + qrow] : -1;
   const int qpos = in ? p.q_pos[(int64_t)b * p.q_len + qrow] : 0;
-  int col_lo = 0, col_hi = 0;
+  int col_lo = 0;
+  unsigned col_width = 0;
   float lse_q = 0.f, delta_q = 0.f;
   if (in && qseg != -1) {
     col_lo = p.dq_mask[0][mbase + qrow / qbs] * kbs;
-    col_hi = p.dq_mask[1][mbase + qrow / qbs] * kbs;
+    col_width = (unsigned)max(p.dq_mask[1][mbase + qrow / qbs] * kbs - col_lo, 0);
     lse_q = p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
     delta_q = p.delta[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
   }
+  TileParts mine[1];
+  mine[0] = wave_parts(col_width > 0, qseg, qpos);
+
+  // live-tile bitmaps over the kv tiles of [t_lo, t_hi)
+  unsigned long long* live = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal);
+  const int word0 = t_lo >> 6;
+  const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
+  const unsigned long long* my_live = live + wave * words;
+  mark_live_tiles<true, 1>(p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles, mine, t_lo, t_hi,
+                           live + wave * words, word0, lane);
+  __syncthreads();
+  int t = next_live_tile<NW>(live, words, word0, t_lo - 1);
 
   f32x16 dq[DT];
 #pragma unroll
@@ -188,7 +199,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
 #pragma unroll
     for (int i = 0; i < 16; i++) dq[dt][i] = 0.f;
 
-  if (t_hi > t_lo) {
+  if (t < t_hi) {
     vec8 qf[KSTEPS], dof[KSTEPS];
     {
       const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
@@ -223,79 +234,62 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
       if (tid < 2 * kTile) reinterpret_cast<int32_t*>(stage + 2 * Smem::kTileBytes)[tid] = idreg;
     };
 
-    load_stage(t_lo * kTile);
+    load_stage(t * kTile);
     store_stage(smem);
     __syncthreads();
 
-    for (int t = t_lo; t < t_hi; t++) {
+    for (int buf = 0; t < t_hi; buf ^= 1) {
       const int kv0 = t * kTile;
-      char* stage = smem + ((t - t_lo) & 1) * Smem::kStage;
-      char* next_stage = smem + ((t - t_lo + 1) & 1) * Smem::kStage;
-      const bool has_next = t + 1 < t_hi;
-      if (has_next) load_stage(kv0 + kTile);
-      const char* ktile = stage;
-      const char* vtile = stage + Smem::kTileBytes;
-      const int32_t* ids = reinterpret_cast<const int32_t*>(stage + 2 * Smem::kTileBytes);
-      const bool full = t >= tf_lo && t < tf_hi;
-      const bool range_test = kv0 < r.max_lo || kv0 + kTile > r.min_hi;
+      char* stage = smem + buf * Smem::kStage;
+      char* next_stage = smem + (buf ^ 1) * Smem::kStage;
+      const int t_next = next_live_tile<NW>(live, words, word0, t);
+      const bool has_next = t_next < t_hi;
+      if (has_next) load_stage(t_next * kTile);
 
-      vec8 dsb[2][2];
+      if (tile_is_live(my_live, word0, t)) {
+        const char* ktile = stage;
+        const char* vtile = stage + Smem::kTileBytes;
+        const int32_t* ids = reinterpret_cast<const int32_t*>(stage + 2 * Smem::kTileBytes);
+        const bool full = t >= tf_lo && t < tf_hi;
+
+        vec8 dsb[2][2];
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++) {
-        f32x16 s, dp;
+        for (int kt = 0; kt < 2; kt++) {
+          f32x16 s, dp;
 #pragma unroll
-        for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
+          for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ks++) {
-          const vec8 ka = read_row8<Tr>(ktile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
-          const vec8 va = read_row8<Tr>(vtile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
-          s = Tr::mfma(ka, qf[ks], s);
-          dp = Tr::mfma(va, dof[ks], dp);
-        }
-#pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-          const int r0 = 32 * kt + 8 * g4 + 4 * h;
-          int sg[4] = {0, 0, 0, 0}, ps[4] = {0, 0, 0, 0};
-          if (!full) {
-            const int4 ksg = *reinterpret_cast<const int4*>(ids + r0);
-            const int4 kps = *reinterpret_cast<const int4*>(ids + kTile + r0);
-            sg[0] = ksg.x, sg[1] = ksg.y, sg[2] = ksg.z, sg[3] = ksg.w;
-            ps[0] = kps.x, ps[1] = kps.y, ps[2] = kps.z, ps[3] = kps.w;
+          for (int ks = 0; ks < KSTEPS; ks++) {
+            const vec8 ka = read_row8<Tr>(ktile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
+            const vec8 va = read_row8<Tr>(vtile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
+            s = Tr::mfma(ka, qf[ks], s);
+            dp = Tr::mfma(va, dof[ks], dp);
           }
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const int i = 4 * g4 + j;
-            float pr = fast_exp2(s[i] * p.scale_log2 - lse_q);
-            if (!full) {
-              bool ok = (sg[j] == qseg) && (qpos >= ps[j]);
-              if (range_test) {
-                const int kv = kv0 + r0 + j;
-                ok = ok && kv >= col_lo && kv < col_hi;
-              } else {
-                ok = ok && col_hi > 0;
-              }
-              if (!ok) pr = 0.f;
+          for (int i = 0; i < 16; i++) s[i] = fast_exp2(__builtin_fmaf(s[i], p.scale_log2, -lse_q));
+          if (!full)
+            mask_c_tile<true>(s, ids, ids + kTile, 32 * kt, kv0, h, qseg, qpos, col_lo, col_width, 0.f);
+#pragma unroll
+          for (int i = 0; i < 16; i++) s[i] *= dp[i] - delta_q;
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+            dsb[kt][st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                                    s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+        }
+        // dQ^T += K^T dS^T
+#pragma unroll
+        for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+              const vec8 a = tr_read_a<Tr>(ktile, Smem::kStride, 32 * kt + 16 * st, 32 * dt, lane);
+              dq[dt] = Tr::mfma(a, dsb[kt][st], dq[dt]);
             }
-            s[i] = pr * (dp[i] - delta_q);
-          }
-        }
-#pragma unroll
-        for (int st = 0; st < 2; st++)
-          dsb[kt][st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
-                                  s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
       }
-      // dQ^T += K^T dS^T
-#pragma unroll
-      for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-        for (int st = 0; st < 2; st++)
-#pragma unroll
-          for (int dt = 0; dt < DT; dt++) {
-            const vec8 a = tr_read_a<Tr>(ktile, Smem::kStride, 32 * kt + 16 * st, 32 * dt, lane);
-            dq[dt] = Tr::mfma(a, dsb[kt][st], dq[dt]);
-          }
       if (has_next) store_stage(next_stage);
       __syncthreads();
+      t = t_next;
     }
   }
 
@@ -356,18 +350,30 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
   const int t_lo = r.lo / kTile;
   const int t_hi = r.hi > r.lo ? (r.hi + kTile - 1) / kTile : t_lo;
   const int tf_lo = (r.flo + kTile - 1) / kTile, tf_hi = r.fhi / kTile;
-  const int nt = t_hi - t_lo;
 
   // per-lane kv column
   const int kvcol = k0 + wave * 32 + c;
   const bool in = kvcol < p.kv_len;
   const int kvseg = in ? p.kv_seg[(int64_t)b * p.kv_len + kvcol] : -1;
   const int kvpos = in ? p.kv_pos[(int64_t)b * p.kv_len + kvcol] : 0;
-  int col_lo = 0, col_hi = 0;
+  int col_lo = 0;
+  unsigned col_width = 0;
   if (in && kvseg != -1) {
     col_lo = p.dkdv_mask[0][mbase + kvcol / kbs] * qbs;
-    col_hi = p.dkdv_mask[1][mbase + kvcol / kbs] * qbs;
+    col_width = (unsigned)max(p.dkdv_mask[1][mbase + kvcol / kbs] * qbs - col_lo, 0);
   }
+  TileParts mine[1];
+  mine[0] = wave_parts(col_width > 0, kvseg, kvpos);
+
+  // live-tile bitmaps over the query tiles of [t_lo, t_hi) (the same for every head of the group)
+  unsigned long long* live = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal);
+  const int word0 = t_lo >> 6;
+  const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
+  const unsigned long long* my_live = live + wave * words;
+  mark_live_tiles<false, 1>(p.q_tiles + 2 * (int64_t)b * p.n_q_tiles, mine, t_lo, t_hi,
+                            live + wave * words, word0, lane);
+  __syncthreads();
+  const int t_first = next_live_tile<NW>(live, words, word0, t_lo - 1);
 
   f32x16 dk[DT], dv[DT];
 #pragma unroll
@@ -375,7 +381,7 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
 #pragma unroll
     for (int i = 0; i < 16; i++) dk[dt][i] = 0.f, dv[dt][i] = 0.f;
 
-  if (nt > 0) {
+  if (t_first < t_hi) {
     vec8 kf[KSTEPS], vf[KSTEPS];
     {
       const char* kr = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh + (int64_t)(in ? kvcol : 0) * p.k_ss) * 2;
@@ -394,9 +400,9 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
 
     RowTile<kTile, D, NT> q_regs, do_regs;
     float rowreg = 0.f;
-    auto load_stage = [&](int step) {
-      const int head = kv_head * p.group + step / nt;
-      const int qr0 = (t_lo + step % nt) * kTile;
+    auto load_stage = [&](int g, int t) {
+      const int head = kv_head * p.group + g;
+      const int qr0 = t * kTile;
       q_regs.load(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, p.q_ss * 2, qr0, p.q_len, tid);
       do_regs.load(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, p.do_ss * 2, qr0, p.q_len, tid);
       if (tid < 4 * kTile) {
@@ -417,89 +423,88 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
       if (tid < 4 * kTile) reinterpret_cast<float*>(stage + 2 * Smem::kTileBytes)[tid] = rowreg;
     };
 
-    const int steps = nt * p.group;
-    load_stage(0);
+    int g = 0, t = t_first;
+    load_stage(g, t);
     store_stage(smem);
     __syncthreads();
 
-    for (int step = 0; step < steps; step++) {
-      const int t = t_lo + step % nt;
+    for (int buf = 0;; buf ^= 1) {
       const int qr0 = t * kTile;
-      char* stage = smem + (step & 1) * Smem::kStage;
-      char* next_stage = smem + ((step + 1) & 1) * Smem::kStage;
-      const bool has_next = step + 1 < steps;
-      if (has_next) load_stage(step + 1);
-      const char* qtile = stage;
-      const char* dotile = stage + Smem::kTileBytes;
-      const float* rowdata = reinterpret_cast<const float*>(stage + 2 * Smem::kTileBytes);
-      const bool full = t >= tf_lo && t < tf_hi;
-      const bool range_test = qr0 < r.max_lo || qr0 + kTile > r.min_hi;
+      char* stage = smem + buf * Smem::kStage;
+      char* next_stage = smem + (buf ^ 1) * Smem::kStage;
+      int t_next = next_live_tile<NW>(live, words, word0, t);
+      int g_next = g;
+      if (t_next >= t_hi) {
+        g_next = g + 1;
+        t_next = t_first;
+      }
+      const bool has_next = g_next < p.group;
+      if (has_next) load_stage(g_next, t_next);
+
+      if (tile_is_live(my_live, word0, t)) {
+        const char* qtile = stage;
+        const char* dotile = stage + Smem::kTileBytes;
+        const float* rowdata = reinterpret_cast<const float*>(stage + 2 * Smem::kTileBytes);
+        const int32_t* rowids = reinterpret_cast<const int32_t*>(rowdata + 2 * kTile);
+        const bool full = t >= tf_lo && t < tf_hi;
 
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++) {
-        f32x16 s, dp;
+        for (int mt = 0; mt < 2; mt++) {
+          f32x16 s, dp;
 #pragma unroll
-        for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
+          for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ks++) {
-          const vec8 qa = read_row8<Tr>(qtile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
-          const vec8 da = read_row8<Tr>(dotile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
-          s = Tr::mfma(qa, kf[ks], s);
-          dp = Tr::mfma(da, vf[ks], dp);
-        }
-        vec8 pb[2], dsb[2];
-#pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-          const int r0 = 32 * mt + 8 * g4 + 4 * h;
-          const float4 lse4 = *reinterpret_cast<const float4*>(rowdata + r0);
-          const float4 del4 = *reinterpret_cast<const float4*>(rowdata + kTile + r0);
-          const float ls[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
-          const float dl[4] = {del4.x, del4.y, del4.z, del4.w};
-          int sg[4] = {0, 0, 0, 0}, ps[4] = {0, 0, 0, 0};
-          if (!full) {
-            const int4 qsg = *reinterpret_cast<const int4*>(rowdata + 2 * kTile + r0);
-            const int4 qps = *reinterpret_cast<const int4*>(rowdata + 3 * kTile + r0);
-            sg[0] = qsg.x, sg[1] = qsg.y, sg[2] = qsg.z, sg[3] = qsg.w;
-            ps[0] = qps.x, ps[1] = qps.y, ps[2] = qps.z, ps[3] = qps.w;
+          for (int ks = 0; ks < KSTEPS; ks++) {
+            const vec8 qa = read_row8<Tr>(qtile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
+            const vec8 da = read_row8<Tr>(dotile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
+            s = Tr::mfma(qa, kf[ks], s);
+            dp = Tr::mfma(da, vf[ks], dp);
           }
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const int i = 4 * g4 + j;
-            float pr = fast_exp2(s[i] * p.scale_log2 - ls[j]);
-            if (!full) {
-              bool ok = (sg[j] == kvseg) && (ps[j] >= kvpos);
-              if (range_test) {
-                const int qi = qr0 + r0 + j;
-                ok = ok && qi >= col_lo && qi < col_hi;
-              } else {
-                ok = ok && col_hi > 0;
-              }
-              if (!ok) pr = 0.f;
+          for (int g4 = 0; g4 < 4; g4++) {
+            const int r0 = 32 * mt + 8 * g4 + 4 * h;
+            const float4 lse4 = *reinterpret_cast<const float4*>(rowdata + r0);
+            const float ls[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+              s[4 * g4 + j] = fast_exp2(__builtin_fmaf(s[4 * g4 + j], p.scale_log2, -ls[j]));
+          }
+          if (!full)
+            mask_c_tile<false>(s, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
+                               col_width, 0.f);
+#pragma unroll
+          for (int g4 = 0; g4 < 4; g4++) {
+            const int r0 = 32 * mt + 8 * g4 + 4 * h;
+            const float4 del4 = *reinterpret_cast<const float4*>(rowdata + kTile + r0);
+            const float dl[4] = {del4.x, del4.y, del4.z, del4.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) dp[4 * g4 + j] = s[4 * g4 + j] * (dp[4 * g4 + j] - dl[j]);
+          }
+          vec8 pb[2], dsb[2];
+#pragma unroll
+          for (int st = 0; st < 2; st++) {
+            pb[st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                               s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+            dsb[st] = pack8<Tr>(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
+                                dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
+          }
+          // dV^T += dO^T P ; dK^T += Q^T dS
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+              const vec8 ad = tr_read_a<Tr>(dotile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
+              dv[dt] = Tr::mfma(ad, pb[st], dv[dt]);
+              const vec8 aq = tr_read_a<Tr>(qtile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
+              dk[dt] = Tr::mfma(aq, dsb[st], dk[dt]);
             }
-            s[i] = pr;
-            dp[i] = pr * (dp[i] - dl[j]);
-          }
         }
-#pragma unroll
-        for (int st = 0; st < 2; st++) {
-          pb[st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
-                             s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
-          dsb[st] = pack8<Tr>(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
-                              dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
-        }
-        // dV^T += dO^T P ; dK^T += Q^T dS
-#pragma unroll
-        for (int st = 0; st < 2; st++)
-#pragma unroll
-          for (int dt = 0; dt < DT; dt++) {
-            const vec8 ad = tr_read_a<Tr>(dotile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
-            dv[dt] = Tr::mfma(ad, pb[st], dv[dt]);
-            const vec8 aq = tr_read_a<Tr>(qtile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
-            dk[dt] = Tr::mfma(aq, dsb[st], dk[dt]);
-          }
       }
       if (has_next) store_stage(next_stage);
       __syncthreads();
+      if (!has_next) break;
+      g = g_next;
+      t = t_next;
     }
   }
 
@@ -536,7 +541,10 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
 }
 
 template <class K>
-int reserve_lds(K kernel, int bytes, bool* done, const char* what) {
+int reserve_lds(K kernel, int need, int bytes, bool* done, const char* what) {
+  if (need > bytes)
+    return fail(KVAX_EUNSUPPORTED, "%s needs %d bytes of LDS for tile bitmaps (limit %d): sequence too long",
+                what, need, bytes);
   if (*done) return KVAX_OK;
   if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
       hipSuccess)
@@ -557,24 +565,32 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
                        dim3(256), 0, stream, p);
     if (int rc = check_launch("fa_bwd_delta_kernel")) return rc;
   }
+  // tile summaries of both sequences (a few microseconds; needed by dQ and dK/dV)
+  {
+    TileSummaryJob jobs[2] = {{p.kv_pos, p.kv_seg, (void*)p.kv_tiles, p.kv_len},
+                              {p.q_pos, p.q_seg, (void*)p.q_tiles, p.q_len}};
+    if (int rc = launch_tile_summaries(jobs, 2, p.batch, stream)) return rc;
+  }
   // dQ
   if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
     auto kernel = fa_bwd_dq_kernel<Tr, D, NW>;
     static bool done = false;
-    if (int rc = reserve_lds(kernel, DqSmem<D>::kTotal, &done, "the dQ kernel")) return rc;
+    const int smem = DqSmem<D>::kTotal + NW * (cdiv(p.n_kv_tiles, 64) + 1) * 8;
+    if (int rc = reserve_lds(kernel, smem, 80 * 1024, &done, "the dQ kernel")) return rc;
     p.num_tiles = cdiv(p.q_len, NW * 32);
     p.total_items = p.batch * p.num_heads * p.num_tiles;
-    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), DqSmem<D>::kTotal, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
   }
   // dK/dV
   if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
     auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW>;
     static bool done = false;
-    if (int rc = reserve_lds(kernel, DkdvSmem<D>::kTotal, &done, "the dK/dV kernel")) return rc;
+    const int smem = DkdvSmem<D>::kTotal + NW * (cdiv(p.n_q_tiles, 64) + 1) * 8;
+    if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, NW * 32);
     p.total_items = p.batch * p.num_kv_heads * p.num_tiles;
-    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), DkdvSmem<D>::kTotal, stream, p);
+    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dkdv_kernel")) return rc;
   }
   return KVAX_OK;
@@ -585,9 +601,14 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
 
 using namespace kvax;
 
+static size_t delta_bytes(const kvax_fa_args* a) {
+  return ((size_t)a->batch * a->num_heads * a->q_len * sizeof(float) + 15) / 16 * 16;
+}
+
 extern "C" size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* a) {
-  if (!a || a->batch < 0 || a->q_len < 0 || a->num_heads < 0) return 0;
-  return (size_t)a->batch * a->num_heads * a->q_len * sizeof(float);  // delta
+  if (!a || a->batch < 0 || a->q_len < 0 || a->kv_len < 0 || a->num_heads < 0) return 0;
+  // delta [batch, heads, q_len] fp32, then the tile summaries of the kv and query sequences
+  return delta_bytes(a) + tile_summary_bytes(a->batch, a->kv_len) + tile_summary_bytes(a->batch, a->q_len);
 }
 
 extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
@@ -617,6 +638,10 @@ extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.dq = (char*)a->dq, p.dk = (char*)a->dk, p.dv = (char*)a->dv;
   p.lse = a->lse;
   p.delta = (float*)workspace;
+  p.kv_tiles = (const int4*)((char*)workspace + delta_bytes(a));
+  p.q_tiles = (const int4*)((char*)workspace + delta_bytes(a) + tile_summary_bytes(a->batch, a->kv_len));
+  p.n_kv_tiles = cdiv(a->kv_len, kTileRows);
+  p.n_q_tiles = cdiv(a->q_len, kTileRows);
   p.q_pos = a->q_pos, p.q_seg = a->q_seg, p.kv_pos = a->kv_pos, p.kv_seg = a->kv_seg;
   for (int i = 0; i < 4; i++) p.dq_mask[i] = a->dq_mask[i], p.dkdv_mask[i] = a->dkdv_mask[i];
   p.q_sb = a->q_strides[0], p.q_ss = a->q_strides[1], p.q_sh = a->q_strides[2];

@@ -121,6 +121,125 @@ __device__ __forceinline__ int xcd_contiguous(int linear, int total) {
 }
 
 
+// ---------------------------------------------------------------------------------------------
+// Tile summaries {seg_min, seg_max, pos_min, pos_max} over non-padding rows (fa_tiles.hip).
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ int4 empty_summary() {
+  return make_int4(0x7fffffff, -0x7fffffff - 1, 0x7fffffff, -0x7fffffff - 1);
+}
+
+// Summary of the rows held one per lane (valid == false lanes are ignored), reduced over the wave.
+__device__ __forceinline__ int4 wave_summary(bool valid, int seg, int pos) {
+  int4 s = empty_summary();
+  if (valid) s = make_int4(seg, seg, pos, pos);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    s.x = min(s.x, __shfl_xor(s.x, off));
+    s.y = max(s.y, __shfl_xor(s.y, off));
+    s.z = min(s.z, __shfl_xor(s.z, off));
+    s.w = max(s.w, __shfl_xor(s.w, off));
+  }
+  return s;
+}
+
+// True when no query of summary `q` can attend any key of summary `k`: segment ranges are
+// disjoint or every key position exceeds every query position.  Empty summaries never attend.
+__device__ __forceinline__ bool cannot_attend(const int4& q, const int4& k) {
+  return (k.y < q.x) | (k.x > q.y) | (k.z > q.w);
+}
+
+// A tile (or a wavefront's own rows) summarised in two parts: rows sharing the segment id of the
+// first non-padding row, and all other non-padding rows.
+struct TileParts {
+  int4 a, b;
+};
+
+__device__ __forceinline__ TileParts wave_parts(bool valid, int seg, int pos) {
+  const unsigned long long vm = __ballot(valid);
+  const int first = vm ? (int)__ffsll((long long)vm) - 1 : 0;
+  const int fseg = __shfl(seg, first);
+  TileParts t;
+  t.a = wave_summary(valid && seg == fseg, seg, pos);
+  t.b = wave_summary(valid && seg != fseg, seg, pos);
+  return t;
+}
+
+__device__ __forceinline__ bool parts_cannot_attend(const TileParts& q, const TileParts& k) {
+  return cannot_attend(q.a, k.a) & cannot_attend(q.a, k.b) & cannot_attend(q.b, k.a) &
+         cannot_attend(q.b, k.b);
+}
+
+// Live-tile bitmaps.  Each wavefront marks, for the tiles [t_lo, t_hi) of the streamed axis, the
+// ones its own rows (NP parts sets) can interact with; bit t % 64 of word t / 64 - word0.
+// `bits` points at this wave's words in LDS.
+template <bool MINE_IS_QUERY, int NP>
+__device__ __forceinline__ void mark_live_tiles(const int4* tiles, const TileParts (&mine)[NP],
+                                                int t_lo, int t_hi, unsigned long long* bits,
+                                                int word0, int lane) {
+  for (int w = word0; w * 64 < t_hi; w++) {
+    const int t = w * 64 + lane;
+    bool live = false;
+    if (t >= t_lo && t < t_hi) {
+      TileParts other;
+      other.a = tiles[2 * t];
+      other.b = tiles[2 * t + 1];
+#pragma unroll
+      for (int i = 0; i < NP; i++)
+        live |= MINE_IS_QUERY ? !parts_cannot_attend(mine[i], other) : !parts_cannot_attend(other, mine[i]);
+    }
+    const unsigned long long m = __ballot(live);
+    if (lane == 0) bits[w - word0] = m;
+  }
+}
+
+// First tile > t_after that is live for any of the NW wavefronts, or INT_MAX.  Uniform.
+template <int NW>
+__device__ __forceinline__ int next_live_tile(const unsigned long long* bits, int words, int word0,
+                                              int t_after) {
+  int t = t_after + 1;
+  int w = max(t >> 6, word0);
+  if (w > (t >> 6)) t = w << 6;
+  while (w - word0 < words) {
+    unsigned long long m = 0;
+#pragma unroll
+    for (int i = 0; i < NW; i++) m |= bits[i * words + (w - word0)];
+    m &= ~0ull << (t & 63);
+    if (m) return (w << 6) + (int)__ffsll((long long)m) - 1;
+    w++;
+    t = w << 6;
+  }
+  return 0x7fffffff;
+}
+
+__device__ __forceinline__ bool tile_is_live(const unsigned long long* wave_bits, int word0, int t) {
+  return (wave_bits[(t >> 6) - word0] >> (t & 63)) & 1;
+}
+
+// Element mask of one 32 x 32 C tile whose columns are per-lane (the wave's own rows) and whose
+// rows are 16 ids of the streamed tile (4 groups of 4 consecutive rows, row_ids = seg[], pos[]).
+// ok = same segment & causal & streamed index inside the column's [c_lo, c_lo + c_width).
+// COL_IS_QUERY: columns are queries (forward, dQ) or keys (dK/dV).  Branch-free.
+template <bool COL_IS_QUERY>
+__device__ __forceinline__ void mask_c_tile(f32x16& s, const int32_t* row_seg, const int32_t* row_pos,
+                                            int row0, int row_global0, int h, int cseg, int cpos,
+                                            int c_lo, unsigned c_width, float fill) {
+#pragma unroll
+  for (int g4 = 0; g4 < 4; g4++) {
+    const int r = row0 + 8 * g4 + 4 * h;
+    const int4 sg = *reinterpret_cast<const int4*>(row_seg + r);
+    const int4 ps = *reinterpret_cast<const int4*>(row_pos + r);
+    const int sgv[4] = {sg.x, sg.y, sg.z, sg.w};
+    const int psv[4] = {ps.x, ps.y, ps.z, ps.w};
+    const int rel = row_global0 + r - c_lo;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const bool causal = COL_IS_QUERY ? (cpos >= psv[j]) : (psv[j] >= cpos);
+      const bool ok = (sgv[j] == cseg) & causal & ((unsigned)(rel + j) < c_width);
+      s[4 * g4 + j] = ok ? s[4 * g4 + j] : fill;
+    }
+  }
+}
+
 // Cooperative staging of a ROWS x D tile of 16-bit elements: global -> registers (issued early
 // so the loads are in flight during compute) -> LDS rows of `lds_stride` bytes.  Rows at or
 // beyond `limit` are zero-filled.

@@ -21,7 +21,7 @@
 namespace kvax {
 namespace {
 
-constexpr int kTK = 64;  // kv rows per LDS tile
+constexpr int kTK = kTileRows;  // kv rows per LDS tile
 
 struct FwdParams {
   const char* q;
@@ -44,7 +44,10 @@ struct FwdParams {
   int batch, q_len, kv_len, num_heads, num_kv_heads, group;
   int qbs, kbs, n_qblocks;
   int num_q_tiles, total_items;
-  float scale_log2;
+  const int4* kv_tiles;  // tile summaries [batch, n_kv_tiles]
+  int n_kv_tiles;
+  uint32_t q_sign;       // 0x80008000 when the scale is negative: Q is negated on load
+  float scale_log2;      // |scale| * log2(e), > 0
 };
 
 template <int D>
@@ -107,8 +110,8 @@ struct TileLoader {
 };
 
 // One work-group: NW wavefronts x (32 * MQ) query rows of one (batch, head); loops over kv tiles.
-template <class Tr, int D, int MQ, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
+template <class Tr, int D, int MQ, int NW, int OCC>
+__global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p) {
   using vec8 = typename Tr::vec8;
   using Smem = FwdSmem<D>;
   constexpr int NT = NW * 64;
@@ -142,27 +145,20 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
   char* obase = p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh) * 2;
   float* lse = p.lse + ((int64_t)b * p.num_heads + head) * p.q_len;
 
-  // ---- kv range of the work-group: union over the mask's query blocks it covers ------------
-  // (element units; the "full" range is the intersection)
+  // ---- kv range of the work-group from the block mask: union of [lower, upper) over the mask's
+  // query blocks it covers, intersection of the full ranges (element units) ---------------------
   int lo = 0x7fffffff, hi = 0, flo = 0, fhi = 0x7fffffff;
-  int min_hi = 0x7fffffff, max_lo = 0;
   {
     const int qb0 = q0 / p.qbs;
     const int qb1 = min((q0 + TQ - 1) / p.qbs, p.n_qblocks - 1);
     for (int qb = qb0; qb <= qb1; qb++) {
       const int64_t mi = (int64_t)b * p.n_qblocks + qb;
       const int l_ = p.lower[mi] * p.kbs, u_ = p.upper[mi] * p.kbs;
-      const int lf = p.lower_full[mi] * p.kbs, uf = p.upper_full[mi] * p.kbs;
-      flo = max(flo, lf);
-      fhi = min(fhi, uf);
+      flo = max(flo, p.lower_full[mi] * p.kbs);
+      fhi = min(fhi, p.upper_full[mi] * p.kbs);
       if (u_ > l_) {
         lo = min(lo, l_);
         hi = max(hi, u_);
-        min_hi = min(min_hi, u_);
-        max_lo = max(max_lo, l_);
-      } else {
-        min_hi = 0;  // a block that attends to nothing: every tile needs the range test
-        max_lo = 0x7fffffff;
       }
     }
   }
@@ -172,20 +168,35 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
   const int tf_lo = (flo + kTK - 1) / kTK, tf_hi = fhi / kTK;
 
   // ---- per-lane query columns ------------------------------------------------------------
-  int qrow[MQ], qseg[MQ], qpos[MQ], col_lo[MQ], col_hi[MQ];
+  int qrow[MQ], qseg[MQ], qpos[MQ], col_lo[MQ];
+  unsigned col_width[MQ];
+  TileParts mine[MQ];
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
     qrow[qt] = q0 + (wave * MQ + qt) * 32 + c;
     const bool in = qrow[qt] < p.q_len;
     qseg[qt] = in ? q_seg[qrow[qt]] : -1;
     qpos[qt] = in ? q_pos[qrow[qt]] : 0;
-    col_lo[qt] = col_hi[qt] = 0;
-    if (in && qseg[qt] != -1) {
+    col_lo[qt] = 0;
+    col_width[qt] = 0;  // padding / out-of-range rows attend to nothing
+    const bool valid = in && qseg[qt] != -1;
+    if (valid) {
       const int64_t mi = (int64_t)b * p.n_qblocks + qrow[qt] / p.qbs;
       col_lo[qt] = p.lower[mi] * p.kbs;
-      col_hi[qt] = p.upper[mi] * p.kbs;
+      col_width[qt] = (unsigned)max(p.upper[mi] * p.kbs - col_lo[qt], 0);
     }
+    mine[qt] = wave_parts(valid && col_width[qt] > 0, qseg[qt], qpos[qt]);
   }
+
+  // ---- live-tile bitmaps: which kv tiles of [t_lo, t_hi) can this wave's rows interact with --
+  unsigned long long* live = reinterpret_cast<unsigned long long*>(smem + 2 * Smem::kStage);
+  const int word0 = t_lo >> 6;
+  const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
+  const unsigned long long* my_live = live + wave * words;
+  mark_live_tiles<true, MQ>(p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles, mine, t_lo, t_hi,
+                            live + wave * words, word0, lane);
+  __syncthreads();
+  int t = next_live_tile<NW>(live, words, word0, t_lo - 1);
 
   f32x16 o[DT][MQ];
   float m_run[MQ], l_run[MQ];
@@ -199,8 +210,9 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
       for (int i = 0; i < 16; i++) o[dt][qt][i] = 0.f;
   }
 
-  if (t_hi > t_lo) {
-    // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step
+  if (t < t_hi) {
+    // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step.
+    // A negative scale is folded into Q so that the softmax below can assume scale_log2 > 0.
     vec8 qf[MQ][KSTEPS];
 #pragma unroll
     for (int qt = 0; qt < MQ; qt++) {
@@ -210,133 +222,115 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
       for (int ks = 0; ks < KSTEPS; ks++) {
         uint4 u = make_uint4(0, 0, 0, 0);
         if (in) u = *reinterpret_cast<const uint4*>(row + (16 * ks + 8 * h) * 2);
+        u.x ^= p.q_sign, u.y ^= p.q_sign, u.z ^= p.q_sign, u.w ^= p.q_sign;
         qf[qt][ks] = __builtin_bit_cast(vec8, u);
       }
     }
+    const float cs = p.scale_log2;  // > 0
 
     TileLoader<D, NT> loader;
-    loader.load(p, kbase, vbase, kv_seg, kv_pos, t_lo * kTK, tid);
+    loader.load(p, kbase, vbase, kv_seg, kv_pos, t * kTK, tid);
     loader.store(smem, tid);
     __syncthreads();
 
-    for (int t = t_lo; t < t_hi; t++) {
+    for (int buf = 0; t < t_hi; buf ^= 1) {
       const int kv0 = t * kTK;
-      char* stage = smem + ((t - t_lo) & 1) * Smem::kStage;
-      char* next_stage = smem + ((t - t_lo + 1) & 1) * Smem::kStage;
-      const bool has_next = t + 1 < t_hi;
-      if (has_next) loader.load(p, kbase, vbase, kv_seg, kv_pos, kv0 + kTK, tid);
+      char* stage = smem + buf * Smem::kStage;
+      char* next_stage = smem + (buf ^ 1) * Smem::kStage;
+      const int t_next = next_live_tile<NW>(live, words, word0, t);
+      const bool has_next = t_next < t_hi;
+      if (has_next) loader.load(p, kbase, vbase, kv_seg, kv_pos, t_next * kTK, tid);
 
-      const char* ktile = stage;
-      const char* vtile = stage + Smem::kKBytes;
-      const int32_t* ids = reinterpret_cast<const int32_t*>(stage + Smem::kKBytes + Smem::kVBytes);
+      if (tile_is_live(my_live, word0, t)) {
+        const char* ktile = stage;
+        const char* vtile = stage + Smem::kKBytes;
+        const int32_t* ids = reinterpret_cast<const int32_t*>(stage + Smem::kKBytes + Smem::kVBytes);
 
-      // ---- S^T = K Q^T -------------------------------------------------------------------
-      f32x16 s[2][MQ];
-#pragma unroll
-      for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-        for (int qt = 0; qt < MQ; qt++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[kt][qt][i] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        vec8 a[2];
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-          a[kt] = read_row8<Tr>(ktile, Smem::kKStride, 32 * kt + c, 16 * ks + 8 * h);
+        // ---- S^T = K Q^T -----------------------------------------------------------------
+        f32x16 s[2][MQ];
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-          for (int qt = 0; qt < MQ; qt++) s[kt][qt] = Tr::mfma(a[kt], qf[qt][ks], s[kt][qt]);
-      }
+          for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[kt][qt][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+          vec8 a[2];
+#pragma unroll
+          for (int kt = 0; kt < 2; kt++)
+            a[kt] = read_row8<Tr>(ktile, Smem::kKStride, 32 * kt + c, 16 * ks + 8 * h);
+#pragma unroll
+          for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int qt = 0; qt < MQ; qt++) s[kt][qt] = Tr::mfma(a[kt], qf[qt][ks], s[kt][qt]);
+        }
 
-      // ---- scale, element mask ------------------------------------------------------------
-      const bool full = t >= tf_lo && t < tf_hi;
-      const bool range_test = kv0 < max_lo || kv0 + kTK > min_hi;
+        // ---- element mask outside the full range (raw scores; masked -> -inf) -------------
+        if (!(t >= tf_lo && t < tf_hi)) {
 #pragma unroll
-      for (int kt = 0; kt < 2; kt++) {
-#pragma unroll
-        for (int qt = 0; qt < MQ; qt++)
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[kt][qt][i] *= p.scale_log2;
-        if (!full) {
-#pragma unroll
-          for (int g4 = 0; g4 < 4; g4++) {
-            const int r0 = 32 * kt + 8 * g4 + 4 * h;
-            const int4 ksg = *reinterpret_cast<const int4*>(ids + r0);
-            const int4 kps = *reinterpret_cast<const int4*>(ids + kTK + r0);
-            const int sg[4] = {ksg.x, ksg.y, ksg.z, ksg.w};
-            const int ps[4] = {kps.x, kps.y, kps.z, kps.w};
+          for (int kt = 0; kt < 2; kt++)
 #pragma unroll
             for (int qt = 0; qt < MQ; qt++)
-#pragma unroll
-              for (int j = 0; j < 4; j++) {
-                bool ok = (sg[j] == qseg[qt]) && (qpos[qt] >= ps[j]);
-                if (range_test) {
-                  const int kv = kv0 + r0 + j;
-                  ok = ok && kv >= col_lo[qt] && kv < col_hi[qt];
-                } else {
-                  ok = ok && col_hi[qt] > 0;
-                }
-                if (!ok) s[kt][qt][4 * g4 + j] = -INFINITY;
-              }
-          }
+              mask_c_tile<true>(s[kt][qt], ids, ids + kTK, 32 * kt, kv0, h, qseg[qt], qpos[qt],
+                                col_lo[qt], col_width[qt], -INFINITY);
         }
-      }
 
-      // ---- online softmax (per query column = per lane, halves combined once) --------------
-      vec8 pb[2][2][MQ];
+        // ---- online softmax (per query column = per lane, halves combined once) ------------
+        vec8 pb[2][2][MQ];
 #pragma unroll
-      for (int qt = 0; qt < MQ; qt++) {
-        float mx = s[0][qt][0];
+        for (int qt = 0; qt < MQ; qt++) {
+          float mx = s[0][qt][0];
+#pragma unroll
+          for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
+          mx = fmaxf(mx, xor32(mx));
+          const float m_new = fmaxf(m_run[qt], mx * cs);
+          if (__any(m_new > m_run[qt])) {
+            const float alpha = fast_exp2(m_run[qt] - m_new);
+            l_run[qt] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+              for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
+          }
+          m_run[qt] = m_new;
+          float sum = 0.f;
+#pragma unroll
+          for (int kt = 0; kt < 2; kt++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+              const float e = fast_exp2(__builtin_fmaf(s[kt][qt][i], cs, -m_new));
+              s[kt][qt][i] = e;
+              sum += e;
+            }
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+              pb[kt][st][qt] = pack8<Tr>(s[kt][qt][8 * st + 0], s[kt][qt][8 * st + 1],
+                                         s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3],
+                                         s[kt][qt][8 * st + 4], s[kt][qt][8 * st + 5],
+                                         s[kt][qt][8 * st + 6], s[kt][qt][8 * st + 7]);
+          }
+          l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
+        }
+
+        // ---- O^T += V^T P^T ---------------------------------------------------------------
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-          for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
-        mx = fmaxf(mx, xor32(mx));
-        const float m_new = fmaxf(m_run[qt], mx);
-        if (__any(m_new > m_run[qt])) {
-          const float alpha = fast_exp2(m_run[qt] - m_new);
-          l_run[qt] *= alpha;
-#pragma unroll
-          for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
-        }
-        m_run[qt] = m_new;
-        float sum = 0.f;
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++) {
-#pragma unroll
-          for (int i = 0; i < 16; i++) {
-            const float e = fast_exp2(s[kt][qt][i] - m_new);
-            s[kt][qt][i] = e;
-            sum += e;
-          }
-#pragma unroll
           for (int st = 0; st < 2; st++)
-            pb[kt][st][qt] = pack8<Tr>(s[kt][qt][8 * st + 0], s[kt][qt][8 * st + 1],
-                                       s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3],
-                                       s[kt][qt][8 * st + 4], s[kt][qt][8 * st + 5],
-                                       s[kt][qt][8 * st + 6], s[kt][qt][8 * st + 7]);
-        }
-        l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) {
+              const vec8 a = tr_read_a<Tr>(vtile, Smem::kVStride, 32 * kt + 16 * st, 32 * dt, lane);
+#pragma unroll
+              for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
+            }
       }
-
-      // ---- O^T += V^T P^T -----------------------------------------------------------------
-#pragma unroll
-      for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-        for (int st = 0; st < 2; st++)
-#pragma unroll
-          for (int dt = 0; dt < DT; dt++) {
-            const vec8 a = tr_read_a<Tr>(vtile, Smem::kVStride, 32 * kt + 16 * st, 32 * dt, lane);
-#pragma unroll
-            for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
-          }
 
       if (has_next) loader.store(next_stage, tid);
       __syncthreads();
+      t = t_next;
     }
   }
 
@@ -344,7 +338,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
     const float l = l_run[qt] + xor32(l_run[qt]);
-    const bool alive = l > 0.f && col_hi[qt] > 0;  // padding / out-of-range rows stay zero
+    const bool alive = l > 0.f && col_width[qt] > 0;  // padding / out-of-range rows stay zero
     const float inv = alive ? 1.f / l : 0.f;
     if (qrow[qt] < p.q_len) {
       char* row = obase + (int64_t)qrow[qt] * p.o_ss * 2;
@@ -362,20 +356,24 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_fwd_kernel(const FwdParams p) {
   }
 }
 
-template <class Tr, int D, int MQ, int NW>
+template <class Tr, int D, int MQ, int NW, int OCC>
 int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   FwdParams p = p0;
   constexpr int TQ = NW * 32 * MQ;
   p.num_q_tiles = cdiv(p.q_len, TQ);
   p.total_items = p.batch * p.num_heads * p.num_q_tiles;
   if (p.total_items == 0) return KVAX_OK;
-  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW>;
-  constexpr int smem = FwdSmem<D>::kTotal;
+  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, OCC>;
+  const int smem = FwdSmem<D>::kTotal + NW * (cdiv(p.n_kv_tiles, 64) + 1) * 8;
+  constexpr int kMaxSmem = 160 * 1024 / OCC;
+  if (smem > kMaxSmem)
+    return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
+                p.kv_len, smem, kMaxSmem);
   static bool configured = false;  // benign race: the attribute is idempotent
   if (!configured) {
-    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem) !=
-        hipSuccess)
-      return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for the forward kernel", smem);
+    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kMaxSmem) != hipSuccess)
+      return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for the forward kernel", kMaxSmem);
     configured = true;
   }
   hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
@@ -413,10 +411,18 @@ int validate_fa_common(const kvax_fa_args* a) {
 
 using namespace kvax;
 
-extern "C" size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args*) { return 0; }
+extern "C" size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* a) {
+  if (!a || a->batch < 0 || a->kv_len < 0) return 0;
+  return tile_summary_bytes(a->batch, a->kv_len);  // kv tile summaries
+}
 
-extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void*, size_t, kvax_stream_t stream_) {
+extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
+                           kvax_stream_t stream_) {
   if (int rc = validate_fa_common(a)) return rc;
+  const size_t need = kvax_fa_fwd_workspace_bytes(a);
+  if (need > workspace_bytes || (need && !workspace))
+    return fail(KVAX_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  if ((uintptr_t)workspace % 16) return fail(KVAX_EINVAL, "workspace must be 16-byte aligned");
   if (a->fwd_query_block <= 0 || a->fwd_kv_block <= 0)
     return fail(KVAX_EINVAL, "forward block sizes must be positive");
   for (int i = 0; i < 4; i++)
@@ -444,11 +450,18 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void*, size_t, kvax_stream_t s
   p.group = a->num_heads / a->num_kv_heads;
   p.qbs = a->fwd_query_block, p.kbs = a->fwd_kv_block;
   p.n_qblocks = cdiv(a->q_len, a->fwd_query_block);
-  p.scale_log2 = a->scale * 1.4426950408889634f;
+  p.q_sign = a->scale < 0.f ? 0x80008000u : 0u;
+  p.scale_log2 = fmaxf(fabsf(a->scale), 1e-30f) * 1.4426950408889634f;
+  p.kv_tiles = (const int4*)workspace;
+  p.n_kv_tiles = cdiv(a->kv_len, kTileRows);
   hipStream_t stream = (hipStream_t)stream_;
   if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
+  {
+    TileSummaryJob job{a->kv_pos, a->kv_seg, workspace, a->kv_len};
+    if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
+  }
   const bool bf16 = a->dtype == KVAX_BF16;
   if (a->head_dim == 128)
-    return bf16 ? launch_fwd<Bf16, 128, 1, 4>(p, stream) : launch_fwd<F16, 128, 1, 4>(p, stream);
-  return bf16 ? launch_fwd<Bf16, 64, 1, 4>(p, stream) : launch_fwd<F16, 64, 1, 4>(p, stream);
+    return bf16 ? launch_fwd<Bf16, 128, 1, 4, 2>(p, stream) : launch_fwd<F16, 128, 1, 4, 2>(p, stream);
+  return bf16 ? launch_fwd<Bf16, 64, 1, 4, 2>(p, stream) : launch_fwd<F16, 64, 1, 4, 2>(p, stream);
 }
