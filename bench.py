@@ -95,7 +95,8 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     from kvax_amd import FlashAttentionParamsConfig, _native, attention_specs, create_attention_mask
-    from kvax_amd.ops.flash_attention import flash_attention_backward, flash_attention_forward
+    from kvax_amd.ops.flash_attention import (backward_workspace_bytes, flash_attention_backward,
+                                              flash_attention_forward)
     from kvax_amd.utils.benchmarking import workload
 
     dev = torch.device("cuda:0")
@@ -131,7 +132,7 @@ def main():
     out = torch.empty_like(q)
     lse = torch.empty((w.batch, w.num_heads, w.q_len), dtype=torch.float32, device=dev)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    ws = torch.empty(w.batch * w.num_heads * w.q_len * 4 + 16, dtype=torch.uint8, device=dev)
+    ws = torch.empty(backward_workspace_bytes(q, k) + 16, dtype=torch.uint8, device=dev)
     SD, SQ, SK = _native.KVAX_FA_SKIP_DELTA, _native.KVAX_FA_SKIP_DQ, _native.KVAX_FA_SKIP_DKDV
 
     def fwd():

@@ -119,24 +119,26 @@ __device__ __forceinline__ Range merged_range(const int32_t* const mask[4], int6
 }
 
 // ---------------------------------------------------------------------------------------------
-// dQ: one work-group = NW wavefronts x 32 query rows of one (batch, head); streams K/V tiles.
+// dQ: one work-group = NW wavefronts x 32 query rows of one (batch, head); streams the live K/V
+// tiles through a ring of LDS stages filled by asynchronous copies.
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int STAGES>
 struct DqSmem {
-  static constexpr int kStride = D * 2 + 16;
-  static constexpr int kTileBytes = kTile * kStride;
+  static constexpr int kTileBytes = kTile * D * 2;  // swizzled, unpadded
   static constexpr int kStage = 2 * kTileBytes + 2 * kTile * 4;
-  static constexpr int kTotal = 2 * kStage;
+  static constexpr int kTotal = STAGES * kStage;
 };
 
-template <class Tr, int D, int NW>
-__global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p) {
+template <class Tr, int D, int NW, int WPS, int STAGES>
+__global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams p) {
   using vec8 = typename Tr::vec8;
-  using Smem = DqSmem<D>;
-  constexpr int NT = NW * 64;
+  using Smem = DqSmem<D, STAGES>;
   constexpr int TQ = NW * 32;
   constexpr int KSTEPS = D / 16;
   constexpr int DT = D / 32;
+  constexpr int RB = D * 2;
+  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
+  static_assert(STAGES == 3, "the loop below keeps two tiles in flight");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -176,22 +178,26 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
   float lse_q = 0.f, delta_q = 0.f;
   if (in && qseg != -1) {
     col_lo = p.dq_mask[0][mbase + qrow / qbs] * kbs;
-    col_width = (unsigned)max(p.dq_mask[1][mbase + qrow / qbs] * kbs - col_lo, 0);
+    col_width = (unsigned)max(min(p.dq_mask[1][mbase + qrow / qbs] * kbs, p.kv_len) - col_lo, 0);
     lse_q = p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
     delta_q = p.delta[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
   }
   TileParts mine[1];
   mine[0] = wave_parts(col_width > 0, qseg, qpos);
 
-  // live-tile bitmaps over the kv tiles of [t_lo, t_hi)
-  unsigned long long* live = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal);
+  // live kv tiles of [t_lo, t_hi): per-wave bitmaps, compacted into one list
+  int* live_count = reinterpret_cast<int*>(smem + Smem::kTotal);
+  unsigned long long* live_bits = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal + 16);
   const int word0 = t_lo >> 6;
   const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
-  const unsigned long long* my_live = live + wave * words;
+  const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.n_kv_tiles, 64) + 1));
   mark_live_tiles<true, 1>(p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles, mine, t_lo, t_hi,
-                           live + wave * words, word0, lane);
+                           live_bits + wave * words, word0, lane);
   __syncthreads();
-  int t = next_live_tile<NW>(live, words, word0, t_lo - 1);
+  if (wave == 0)
+    compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
+  __syncthreads();
+  const int n_live = *live_count;
 
   f32x16 dq[DT];
 #pragma unroll
@@ -199,7 +205,7 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
 #pragma unroll
     for (int i = 0; i < 16; i++) dq[dt][i] = 0.f;
 
-  if (t < t_hi) {
+  if (n_live > 0) {
     vec8 qf[KSTEPS], dof[KSTEPS];
     {
       const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
@@ -215,41 +221,44 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
         dof[ks] = __builtin_bit_cast(vec8, w);
       }
     }
+    int nat_off[KSTEPS], tr_off[DT][2];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) nat_off[ks] = nat_offset<D>(c, ks, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      tr_off[dt][0] = tr_offset<D>(lane, dt, 0);
+      tr_off[dt][1] = tr_offset<D>(lane, dt, 1);
+    }
 
-    RowTile<kTile, D, NT> kt_regs, vt_regs;
-    int32_t idreg = 0;
-    auto load_stage = [&](int kv0) {
-      kt_regs.load(kbase, p.k_ss * 2, kv0, p.kv_len, tid);
-      vt_regs.load(vbase, p.v_ss * 2, kv0, p.kv_len, tid);
-      if (tid < 2 * kTile) {
-        const int kv = kv0 + tid % kTile;
-        const bool is_seg = tid < kTile;
-        idreg = is_seg ? -1 : 0;
-        if (kv < p.kv_len) idreg = is_seg ? kv_seg[kv] : kv_pos[kv];
-      }
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
+    const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
+    auto issue = [&](int tile, int stage) {
+      const uint32_t base = smem_addr + stage * Smem::kStage;
+      async_tile_copy<kTile, D, NW>(kbase, p.k_ss * 2, tile * kTile, p.kv_len, base, wave, lane);
+      async_tile_copy<kTile, D, NW>(vbase, p.v_ss * 2, tile * kTile, p.kv_len, base + Smem::kTileBytes, wave, lane);
+      async_copy_b32(id_src + min(tile * kTile + lane, p.kv_len - 1),
+                     __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + (wave & 1) * (kTile * 4)));
     };
-    auto store_stage = [&](char* stage) {
-      kt_regs.store(stage, Smem::kStride, tid);
-      vt_regs.store(stage + Smem::kTileBytes, Smem::kStride, tid);
-      if (tid < 2 * kTile) reinterpret_cast<int32_t*>(stage + 2 * Smem::kTileBytes)[tid] = idreg;
-    };
 
-    load_stage(t * kTile);
-    store_stage(smem);
-    __syncthreads();
+    uint32_t e0 = live_list[0];
+    uint32_t e1 = n_live > 1 ? live_list[1] : 0;
+    uint32_t e2 = n_live > 2 ? live_list[2] : 0;
+    issue(e0 & 0xffffff, 0);
+    if (n_live > 1) issue(e1 & 0xffffff, 1);
 
-    for (int buf = 0; t < t_hi; buf ^= 1) {
-      const int kv0 = t * kTile;
-      char* stage = smem + buf * Smem::kStage;
-      char* next_stage = smem + (buf ^ 1) * Smem::kStage;
-      const int t_next = next_live_tile<NW>(live, words, word0, t);
-      const bool has_next = t_next < t_hi;
-      if (has_next) load_stage(t_next * kTile);
+    int stage = 0;
+    for (int i = 0; i < n_live; i++) {
+      if (i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      __syncthreads();
+      const uint32_t e3 = i + 3 < n_live ? live_list[i + 3] : 0;
+      if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      const int t = e0 & 0xffffff;
 
-      if (tile_is_live(my_live, word0, t)) {
-        const char* ktile = stage;
-        const char* vtile = stage + Smem::kTileBytes;
-        const int32_t* ids = reinterpret_cast<const int32_t*>(stage + 2 * Smem::kTileBytes);
+      if ((e0 >> (24 + wave)) & 1) {
+        const int kv0 = t * kTile;
+        const char* ktile = smem + stage * Smem::kStage;
+        const char* vtile = ktile + Smem::kTileBytes;
+        const int32_t* ids = reinterpret_cast<const int32_t*>(ktile + 2 * Smem::kTileBytes);
         const bool full = t >= tf_lo && t < tf_hi;
 
         vec8 dsb[2][2];
@@ -257,20 +266,20 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
         for (int kt = 0; kt < 2; kt++) {
           f32x16 s, dp;
 #pragma unroll
-          for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
+          for (int i2 = 0; i2 < 16; i2++) s[i2] = 0.f, dp[i2] = 0.f;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ks++) {
-            const vec8 ka = read_row8<Tr>(ktile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
-            const vec8 va = read_row8<Tr>(vtile, Smem::kStride, 32 * kt + c, 16 * ks + 8 * h);
+            const vec8 ka = *reinterpret_cast<const vec8*>(ktile + 32 * kt * RB + nat_off[ks]);
+            const vec8 va = *reinterpret_cast<const vec8*>(vtile + 32 * kt * RB + nat_off[ks]);
             s = Tr::mfma(ka, qf[ks], s);
             dp = Tr::mfma(va, dof[ks], dp);
           }
 #pragma unroll
-          for (int i = 0; i < 16; i++) s[i] = fast_exp2(__builtin_fmaf(s[i], p.scale_log2, -lse_q));
+          for (int i2 = 0; i2 < 16; i2++) s[i2] = fast_exp2(__builtin_fmaf(s[i2], p.scale_log2, -lse_q));
           if (!full)
             mask_c_tile<true>(s, ids, ids + kTile, 32 * kt, kv0, h, qseg, qpos, col_lo, col_width, 0.f);
 #pragma unroll
-          for (int i = 0; i < 16; i++) s[i] *= dp[i] - delta_q;
+          for (int i2 = 0; i2 < 16; i2++) s[i2] *= dp[i2] - delta_q;
 #pragma unroll
           for (int st = 0; st < 2; st++)
             dsb[kt][st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
@@ -283,13 +292,12 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-              const vec8 a = tr_read_a<Tr>(ktile, Smem::kStride, 32 * kt + 16 * st, 32 * dt, lane);
+              const vec8 a = tr_read_a_swz<Tr>(ktile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
               dq[dt] = Tr::mfma(a, dsb[kt][st], dq[dt]);
             }
       }
-      if (has_next) store_stage(next_stage);
-      __syncthreads();
-      t = t_next;
+      e0 = e1, e1 = e2, e2 = e3;
+      stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
   }
 
@@ -308,27 +316,28 @@ __global__ __launch_bounds__(NW * 64, 2) void fa_bwd_dq_kernel(const BwdParams p
 }
 
 // ---------------------------------------------------------------------------------------------
-// dK/dV: one work-group = NW wavefronts x 32 kv rows of one (batch, kv head); streams the Q / dO
-// tiles of every query head of the group and accumulates dK^T, dV^T in registers.
+// dK/dV: one work-group = NW wavefronts x 32 kv rows of one (batch, kv head); streams the live
+// Q / dO tiles of every query head of the group and accumulates dK^T, dV^T in registers.
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int STAGES>
 struct DkdvSmem {
-  static constexpr int kStride = D * 2 + 16;
-  static constexpr int kTileBytes = kTile * kStride;
-  static constexpr int kRowData = 4 * kTile * 4;  // lse, delta, seg, pos
+  static constexpr int kTileBytes = kTile * D * 2;  // swizzled, unpadded
+  static constexpr int kRowData = 4 * kTile * 4;    // lse, delta, seg, pos
   static constexpr int kStage = 2 * kTileBytes + kRowData;
-  static constexpr int kTotal = 2 * kStage;
+  static constexpr int kTotal = STAGES * kStage;
 };
 
-template <class Tr, int D, int NW>
-__global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams p) {
+template <class Tr, int D, int NW, int WPS, int STAGES>
+__global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdParams p) {
   using vec8 = typename Tr::vec8;
-  using Smem = DkdvSmem<D>;
-  constexpr int NT = NW * 64;
+  using Smem = DkdvSmem<D, STAGES>;
   constexpr int TKV = NW * 32;
   constexpr int KSTEPS = D / 16;
   constexpr int DT = D / 32;
-  static_assert(NT >= 4 * kTile, "row data is staged by one thread per value");
+  constexpr int RB = D * 2;
+  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
+  static_assert(STAGES == 3, "the loop below keeps two tiles in flight");
+  static_assert(NW >= 4 && NW % 4 == 0, "one wave per row-data array");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -360,20 +369,26 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
   unsigned col_width = 0;
   if (in && kvseg != -1) {
     col_lo = p.dkdv_mask[0][mbase + kvcol / kbs] * qbs;
-    col_width = (unsigned)max(p.dkdv_mask[1][mbase + kvcol / kbs] * qbs - col_lo, 0);
+    // queries at or beyond q_len never count (their LDS rows hold a copy of the last row)
+    col_width = (unsigned)max(min(p.dkdv_mask[1][mbase + kvcol / kbs] * qbs, p.q_len) - col_lo, 0);
   }
   TileParts mine[1];
   mine[0] = wave_parts(col_width > 0, kvseg, kvpos);
 
-  // live-tile bitmaps over the query tiles of [t_lo, t_hi) (the same for every head of the group)
-  unsigned long long* live = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal);
+  // live query tiles of [t_lo, t_hi) (the same for every head of the group)
+  int* live_count = reinterpret_cast<int*>(smem + Smem::kTotal);
+  unsigned long long* live_bits = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal + 16);
   const int word0 = t_lo >> 6;
   const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
-  const unsigned long long* my_live = live + wave * words;
+  const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.n_q_tiles, 64) + 1));
   mark_live_tiles<false, 1>(p.q_tiles + 2 * (int64_t)b * p.n_q_tiles, mine, t_lo, t_hi,
-                            live + wave * words, word0, lane);
+                            live_bits + wave * words, word0, lane);
   __syncthreads();
-  const int t_first = next_live_tile<NW>(live, words, word0, t_lo - 1);
+  if (wave == 0)
+    compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
+  __syncthreads();
+  const int n_live = *live_count;
+  const int steps = n_live * p.group;  // every head of the group walks the same list
 
   f32x16 dk[DT], dv[DT];
 #pragma unroll
@@ -381,7 +396,7 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
 #pragma unroll
     for (int i = 0; i < 16; i++) dk[dt][i] = 0.f, dv[dt][i] = 0.f;
 
-  if (t_first < t_hi) {
+  if (steps > 0) {
     vec8 kf[KSTEPS], vf[KSTEPS];
     {
       const char* kr = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh + (int64_t)(in ? kvcol : 0) * p.k_ss) * 2;
@@ -397,54 +412,55 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
         vf[ks] = __builtin_bit_cast(vec8, w);
       }
     }
+    int nat_off[KSTEPS], tr_off[DT][2];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) nat_off[ks] = nat_offset<D>(c, ks, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      tr_off[dt][0] = tr_offset<D>(lane, dt, 0);
+      tr_off[dt][1] = tr_offset<D>(lane, dt, 1);
+    }
 
-    RowTile<kTile, D, NT> q_regs, do_regs;
-    float rowreg = 0.f;
-    auto load_stage = [&](int g, int t) {
-      const int head = kv_head * p.group + g;
-      const int qr0 = t * kTile;
-      q_regs.load(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, p.q_ss * 2, qr0, p.q_len, tid);
-      do_regs.load(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, p.do_ss * 2, qr0, p.q_len, tid);
-      if (tid < 4 * kTile) {
-        const int which = tid / kTile;
-        const int qi = qr0 + tid % kTile;
-        const bool ok = qi < p.q_len;
-        const int64_t hoff = ((int64_t)b * p.num_heads + head) * p.q_len + qi;
-        const int64_t boff = (int64_t)b * p.q_len + qi;
-        if (which == 0) rowreg = ok ? p.lse[hoff] : 0.f;
-        else if (which == 1) rowreg = ok ? p.delta[hoff] : 0.f;
-        else if (which == 2) rowreg = __int_as_float(ok ? p.q_seg[boff] : -1);
-        else rowreg = __int_as_float(ok ? p.q_pos[boff] : 0);
-      }
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
+    const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos
+    // step s = (head s / n_live of the group, list entry s % n_live)
+    auto issue = [&](int step, uint32_t entry, int stage) {
+      const int head = kv_head * p.group + step / n_live;
+      const int qr0 = (int)(entry & 0xffffff) * kTile;
+      const uint32_t base = smem_addr + stage * Smem::kStage;
+      async_tile_copy<kTile, D, NW>(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, p.q_ss * 2, qr0,
+                                    p.q_len, base, wave, lane);
+      async_tile_copy<kTile, D, NW>(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, p.do_ss * 2,
+                                    qr0, p.q_len, base + Smem::kTileBytes, wave, lane);
+      const int qi = min(qr0 + lane, p.q_len - 1);
+      const int64_t hoff = ((int64_t)b * p.num_heads + head) * p.q_len + qi;
+      const int64_t boff = (int64_t)b * p.q_len + qi;
+      const void* src = which == 0 ? (const void*)(p.lse + hoff)
+                      : which == 1 ? (const void*)(p.delta + hoff)
+                      : which == 2 ? (const void*)(p.q_seg + boff) : (const void*)(p.q_pos + boff);
+      async_copy_b32(src, __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + which * (kTile * 4)));
     };
-    auto store_stage = [&](char* stage) {
-      q_regs.store(stage, Smem::kStride, tid);
-      do_regs.store(stage + Smem::kTileBytes, Smem::kStride, tid);
-      if (tid < 4 * kTile) reinterpret_cast<float*>(stage + 2 * Smem::kTileBytes)[tid] = rowreg;
-    };
+    auto entry_of = [&](int step) { return live_list[step % n_live]; };
 
-    int g = 0, t = t_first;
-    load_stage(g, t);
-    store_stage(smem);
-    __syncthreads();
+    uint32_t e0 = entry_of(0);
+    uint32_t e1 = steps > 1 ? entry_of(1) : 0;
+    uint32_t e2 = steps > 2 ? entry_of(2) : 0;
+    issue(0, e0, 0);
+    if (steps > 1) issue(1, e1, 1);
 
-    for (int buf = 0;; buf ^= 1) {
-      const int qr0 = t * kTile;
-      char* stage = smem + buf * Smem::kStage;
-      char* next_stage = smem + (buf ^ 1) * Smem::kStage;
-      int t_next = next_live_tile<NW>(live, words, word0, t);
-      int g_next = g;
-      if (t_next >= t_hi) {
-        g_next = g + 1;
-        t_next = t_first;
-      }
-      const bool has_next = g_next < p.group;
-      if (has_next) load_stage(g_next, t_next);
+    int stage = 0;
+    for (int step = 0; step < steps; step++) {
+      if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      __syncthreads();
+      const uint32_t e3 = step + 3 < steps ? entry_of(step + 3) : 0;
+      if (step + 2 < steps) issue(step + 2, e2, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      const int t = e0 & 0xffffff;
 
-      if (tile_is_live(my_live, word0, t)) {
-        const char* qtile = stage;
-        const char* dotile = stage + Smem::kTileBytes;
-        const float* rowdata = reinterpret_cast<const float*>(stage + 2 * Smem::kTileBytes);
+      if ((e0 >> (24 + wave)) & 1) {
+        const int qr0 = t * kTile;
+        const char* qtile = smem + stage * Smem::kStage;
+        const char* dotile = qtile + Smem::kTileBytes;
+        const float* rowdata = reinterpret_cast<const float*>(qtile + 2 * Smem::kTileBytes);
         const int32_t* rowids = reinterpret_cast<const int32_t*>(rowdata + 2 * kTile);
         const bool full = t >= tf_lo && t < tf_hi;
 
@@ -455,8 +471,8 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
           for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
 #pragma unroll
           for (int ks = 0; ks < KSTEPS; ks++) {
-            const vec8 qa = read_row8<Tr>(qtile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
-            const vec8 da = read_row8<Tr>(dotile, Smem::kStride, 32 * mt + c, 16 * ks + 8 * h);
+            const vec8 qa = *reinterpret_cast<const vec8*>(qtile + 32 * mt * RB + nat_off[ks]);
+            const vec8 da = *reinterpret_cast<const vec8*>(dotile + 32 * mt * RB + nat_off[ks]);
             s = Tr::mfma(qa, kf[ks], s);
             dp = Tr::mfma(da, vf[ks], dp);
           }
@@ -493,18 +509,15 @@ __global__ __launch_bounds__(NW * 64, 1) void fa_bwd_dkdv_kernel(const BwdParams
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-              const vec8 ad = tr_read_a<Tr>(dotile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
+              const vec8 ad = tr_read_a_swz<Tr>(dotile + (32 * mt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
               dv[dt] = Tr::mfma(ad, pb[st], dv[dt]);
-              const vec8 aq = tr_read_a<Tr>(qtile, Smem::kStride, 32 * mt + 16 * st, 32 * dt, lane);
+              const vec8 aq = tr_read_a_swz<Tr>(qtile + (32 * mt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
               dk[dt] = Tr::mfma(aq, dsb[st], dk[dt]);
             }
         }
       }
-      if (has_next) store_stage(next_stage);
-      __syncthreads();
-      if (!has_next) break;
-      g = g_next;
-      t = t_next;
+      e0 = e1, e1 = e2, e2 = e3;
+      stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
   }
 
@@ -555,14 +568,14 @@ int reserve_lds(K kernel, int need, int bytes, bool* done, const char* what) {
 
 template <class Tr, int D>
 int launch_bwd(BwdParams p, hipStream_t stream) {
-  constexpr int NW = 4;
+  constexpr int STAGES = 3;
   // delta
   if (!(p.flags & KVAX_FA_SKIP_DELTA)) {
     const int64_t rows = (int64_t)p.batch * p.q_len * p.num_heads;
     constexpr int kRowsPerGroup = 256 / (D / 8);
     if (rows > 0)
       hipLaunchKernelGGL((fa_bwd_delta_kernel<Tr, D>), dim3((unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup)),
-                       dim3(256), 0, stream, p);
+                         dim3(256), 0, stream, p);
     if (int rc = check_launch("fa_bwd_delta_kernel")) return rc;
   }
   // tile summaries of both sequences (a few microseconds; needed by dQ and dK/dV)
@@ -571,22 +584,24 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
                               {p.q_pos, p.q_seg, (void*)p.q_tiles, p.q_len}};
     if (int rc = launch_tile_summaries(jobs, 2, p.batch, stream)) return rc;
   }
-  // dQ
+  // dQ: 8 wavefronts (256 query rows) per work-group, two per SIMD, one work-group per CU
   if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
-    auto kernel = fa_bwd_dq_kernel<Tr, D, NW>;
+    constexpr int NW = 8;
+    auto kernel = fa_bwd_dq_kernel<Tr, D, NW, 2, STAGES>;
     static bool done = false;
-    const int smem = DqSmem<D>::kTotal + NW * (cdiv(p.n_kv_tiles, 64) + 1) * 8;
-    if (int rc = reserve_lds(kernel, smem, 80 * 1024, &done, "the dQ kernel")) return rc;
+    const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
+    if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dQ kernel")) return rc;
     p.num_tiles = cdiv(p.q_len, NW * 32);
     p.total_items = p.batch * p.num_heads * p.num_tiles;
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
   }
-  // dK/dV
+  // dK/dV: 4 wavefronts (128 kv rows) per work-group, one per SIMD
   if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
-    auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW>;
+    constexpr int NW = 4;
+    auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW, 1, STAGES>;
     static bool done = false;
-    const int smem = DkdvSmem<D>::kTotal + NW * (cdiv(p.n_q_tiles, 64) + 1) * 8;
+    const int smem = DkdvSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
     if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, NW * 32);
     p.total_items = p.batch * p.num_kv_heads * p.num_tiles;

@@ -109,6 +109,8 @@ __device__ __forceinline__ typename Tr::vec8 read_row8(const char* tile, int str
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+__device__ __forceinline__ int cdiv_dev(int a, int b) { return (a + b - 1) / b; }
+
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32); }
 
 // Work-group index -> work item, so that each XCD (work-groups are dealt round-robin to the 8
@@ -215,6 +217,35 @@ __device__ __forceinline__ bool tile_is_live(const unsigned long long* wave_bits
   return (wave_bits[(t >> 6) - word0] >> (t & 63)) & 1;
 }
 
+// Compacts the NW per-wave bitmaps into a list of the tiles that are live for at least one
+// wavefront: entry = tile index | (mask of the waves it is live for) << 24.  Executed by one
+// wavefront; the number of entries is written to *count.
+template <int NW>
+__device__ __forceinline__ void compact_live_tiles(const unsigned long long* bits, int words, int word0,
+                                                   uint32_t* list, int* count, int lane) {
+  static_assert(NW <= 8, "the wave mask is stored in the top byte of an entry");
+  int n = 0;
+  for (int w = 0; w < words; w++) {
+    unsigned long long any = 0;
+    uint32_t waves = 0;
+#pragma unroll
+    for (int i = 0; i < NW; i++) {
+      const unsigned long long m = bits[i * words + w];
+      any |= m;
+      waves |= (uint32_t)((m >> lane) & 1) << i;
+    }
+    if ((any >> lane) & 1)
+      list[n + __popcll(any & ((1ull << lane) - 1))] = (uint32_t)((word0 + w) * 64 + lane) | (waves << 24);
+    n += __popcll(any);
+  }
+  if (lane == 0) *count = n;
+}
+
+// LDS bytes for the live-tile bookkeeping of a range of at most `tiles` tiles.
+__host__ __device__ constexpr int live_tiles_bytes(int nw, int tiles) {
+  return 16 + nw * ((tiles + 63) / 64 + 1) * 8 + tiles * 4;
+}
+
 // Element mask of one 32 x 32 C tile whose columns are per-lane (the wave's own rows) and whose
 // rows are 16 ids of the streamed tile (4 groups of 4 consecutive rows, row_ids = seg[], pos[]).
 // ok = same segment & causal & streamed index inside the column's [c_lo, c_lo + c_width).
@@ -238,6 +269,95 @@ __device__ __forceinline__ void mask_c_tile(f32x16& s, const int32_t* row_seg, c
       s[4 * g4 + j] = ok ? s[4 * g4 + j] : fill;
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Swizzled LDS tiles filled by asynchronous global -> LDS copies.
+//
+// A tile is ROWS rows of D 16-bit elements, unpadded (D * 2 bytes per row).  The 16-byte chunk c
+// of row r lives at chunk position c ^ swz<D>(r).  With this permutation both access patterns
+// of the kernels are bank-conflict free on the same tile: row reads (16 lanes = 16 consecutive
+// rows, one chunk each) and 4-row transposing reads (ds_read_b64_tr_b16).  Unpadded rows also
+// make each 1 KiB of the tile contiguous, which is what a wave-wide global_load_lds_dwordx4
+// writes (lane i -> LDS base + 16 * i), so tiles are copied without passing through registers.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ int swz(int r) {
+  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);  // D == 64: 8 chunks per row
+}
+
+// One asynchronous 16-byte-per-lane copy: the wave writes 1 KiB at LDS address `lds_addr`
+// (wave-uniform), lane i providing its own global source address.  Completion is tracked by
+// vmcnt; the data is visible to other waves after an s_waitcnt vmcnt + barrier.  Issued through
+// inline assembly so that the compiler does not serialise later LDS reads against it.
+__device__ __forceinline__ void async_copy_b128(const void* gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr)
+               : "memory");
+}
+// Same for 4 bytes per lane (256 B per wave).
+__device__ __forceinline__ void async_copy_b32(const void* gptr, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_addr), "v"(gptr)
+               : "memory");
+}
+
+// s_waitcnt vmcnt(N) leaving the other counters alone (gfx9 encoding: vmcnt = bits 3:0 and
+// 15:14, expcnt = 6:4, lgkmcnt = 11:8).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// Copies rows [row0, row0 + ROWS) of a row-major global matrix (16-bit elements, D per row,
+// `row_stride_bytes` between rows) into a swizzled LDS tile at LDS address `tile_addr`.  Rows at
+// or beyond `limit` (>= 1) are replaced by row limit - 1: callers mask them out by index.
+// Every wave issues ROWS * D * 2 / 1024 / NW copies.
+template <int ROWS, int D, int NW>
+__device__ __forceinline__ void async_tile_copy(const char* gbase, int64_t row_stride_bytes, int row0,
+                                                int limit, uint32_t tile_addr, int wave, int lane) {
+  constexpr int kRowsPerCopy = 1024 / (D * 2);  // 4 (D = 128) or 8 (D = 64)
+  constexpr int kCopies = ROWS / kRowsPerCopy;
+  constexpr int kChunks = D / 8;
+  static_assert(kCopies % NW == 0, "copies must split evenly over the waves");
+  const int rin = lane / kChunks, pos = lane % kChunks;
+#pragma unroll
+  for (int j = 0; j < kCopies / NW; j++) {
+    const int grp = j * NW + wave;
+    const int r = grp * kRowsPerCopy + rin;
+    const int chunk = pos ^ swz<D>(r);
+    const int grow = min(row0 + r, limit - 1);
+    async_copy_b128(gbase + (int64_t)grow * row_stride_bytes + chunk * 16,
+                    __builtin_amdgcn_readfirstlane(tile_addr + grp * 1024));
+  }
+}
+template <int ROWS, int D, int NW>
+constexpr int async_tile_copies_per_wave() {
+  return ROWS / (1024 / (D * 2)) / NW;
+}
+
+// Per-lane byte offsets into a swizzled tile.
+// Row read (natural MFMA operand): lane (c, h) reads elements [16 * ks + 8 * h, +8) of row
+// `row_in_16 + 32 * kt`; nat_offset gives the offset for kt = 0, add 32 * kt * D * 2.
+template <int D>
+__device__ __forceinline__ int nat_offset(int row, int ks, int h) {
+  return row * (D * 2) + ((((2 * ks) | h) ^ swz<D>(row)) << 4);
+}
+// Transposed operand gather (see tr_read_a): lane (g, i) of step `half` (0: first 4-row read,
+// 1: second) for the 32-column block dt; add row0 * D * 2 for the row block (row0 % 16 == 0).
+template <int D>
+__device__ __forceinline__ int tr_offset(int lane, int dt, int half) {
+  const int g = lane >> 4, i = lane & 15;
+  const int row = 4 * (g >> 1) + (i >> 2) + 8 * half;
+  const int chunk = 4 * dt + 2 * (g & 1) + ((i & 3) >> 1);
+  return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4) + (i & 1) * 8;
+}
+template <class Tr>
+__device__ __forceinline__ typename Tr::vec8 tr_read_a_swz(const char* tile_row0, int off_lo, int off_hi) {
+  s16x4 lo = ds_read_tr16(tile_row0 + off_lo);
+  s16x4 hi = ds_read_tr16(tile_row0 + off_hi);
+  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(typename Tr::vec8, v);
 }
 
 // Cooperative staging of a ROWS x D tile of 16-bit elements: global -> registers (issued early

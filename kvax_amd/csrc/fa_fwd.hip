@@ -15,6 +15,8 @@
 // staged through LDS once per work-group (double buffered, prefetched through registers) and
 // shared by the work-group's wavefronts; the query heads of one GQA group run as neighbouring
 // work-groups on one XCD so K/V tiles are served from that XCD's L2.
+#include <cstdlib>
+
 #include "common.h"
 #include "fa_common.h"
 
@@ -50,74 +52,26 @@ struct FwdParams {
   float scale_log2;      // |scale| * log2(e), > 0
 };
 
-template <int D>
+template <int D, int STAGES>
 struct FwdSmem {
-  static constexpr int kKStride = D * 2 + 16;  // bytes; 16 B pad => conflict-free b128 row reads
-  static constexpr int kVStride = D * 2 + 64;  // bytes; 64 B pad spreads the 4-row tr reads
-  static constexpr int kKBytes = kTK * kKStride;
-  static constexpr int kVBytes = kTK * kVStride;
-  static constexpr int kIdBytes = 2 * kTK * 4;  // seg + pos
-  static constexpr int kStage = kKBytes + kVBytes + kIdBytes;
-  static constexpr int kTotal = 2 * kStage;
+  static constexpr int kTileBytes = kTK * D * 2;  // swizzled, unpadded
+  static constexpr int kIdBytes = 2 * kTK * 4;    // seg + pos
+  static constexpr int kStage = 2 * kTileBytes + kIdBytes;
+  static constexpr int kTotal = STAGES * kStage;
 };
 
-// Cooperative global -> register -> LDS staging of one K/V tile (+ its ids).
-template <int D, int NT>
-struct TileLoader {
-  static constexpr int kChunksPerRow = D / 8;                    // 16-byte chunks
-  static constexpr int kPerThread = kTK * kChunksPerRow / NT;    // chunks per thread per tensor
-  static_assert(kTK * kChunksPerRow % NT == 0, "tile must split evenly over the work-group");
-  uint4 kreg[kPerThread];
-  uint4 vreg[kPerThread];
-  int32_t idreg;
-
-  __device__ __forceinline__ void load(const FwdParams& p, const char* kbase, const char* vbase,
-                                       const int32_t* seg, const int32_t* pos, int kv0, int tid) {
-#pragma unroll
-    for (int i = 0; i < kPerThread; i++) {
-      const int id = tid + i * NT;
-      const int row = id / kChunksPerRow, ch = id % kChunksPerRow;
-      const int kv = kv0 + row;
-      if (kv < p.kv_len) {
-        kreg[i] = *reinterpret_cast<const uint4*>(kbase + (int64_t)kv * p.k_ss * 2 + ch * 16);
-        vreg[i] = *reinterpret_cast<const uint4*>(vbase + (int64_t)kv * p.v_ss * 2 + ch * 16);
-      } else {
-        kreg[i] = make_uint4(0, 0, 0, 0);
-        vreg[i] = make_uint4(0, 0, 0, 0);
-      }
-    }
-    if (tid < 2 * kTK) {
-      const int kv = kv0 + (tid % kTK);
-      const bool is_seg = tid < kTK;
-      idreg = is_seg ? -1 : 0;
-      if (kv < p.kv_len) idreg = is_seg ? seg[kv] : pos[kv];
-    }
-  }
-
-  __device__ __forceinline__ void store(char* stage, int tid) {
-    char* kt = stage;
-    char* vt = stage + FwdSmem<D>::kKBytes;
-#pragma unroll
-    for (int i = 0; i < kPerThread; i++) {
-      const int id = tid + i * NT;
-      const int row = id / kChunksPerRow, ch = id % kChunksPerRow;
-      *reinterpret_cast<uint4*>(kt + row * FwdSmem<D>::kKStride + ch * 16) = kreg[i];
-      *reinterpret_cast<uint4*>(vt + row * FwdSmem<D>::kVStride + ch * 16) = vreg[i];
-    }
-    if (tid < 2 * kTK)
-      reinterpret_cast<int32_t*>(stage + FwdSmem<D>::kKBytes + FwdSmem<D>::kVBytes)[tid] = idreg;
-  }
-};
-
-// One work-group: NW wavefronts x (32 * MQ) query rows of one (batch, head); loops over kv tiles.
-template <class Tr, int D, int MQ, int NW, int OCC>
-__global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p) {
+// One work-group: NW wavefronts x (32 * MQ) query rows of one (batch, head); streams the live kv
+// tiles through a STAGES-deep ring of LDS stages filled by asynchronous copies.
+template <class Tr, int D, int MQ, int NW, int WPS, int STAGES>
+__global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p) {
   using vec8 = typename Tr::vec8;
-  using Smem = FwdSmem<D>;
-  constexpr int NT = NW * 64;
+  using Smem = FwdSmem<D, STAGES>;
   constexpr int TQ = NW * 32 * MQ;
   constexpr int KSTEPS = D / 16;  // contraction steps of S^T = K Q^T
   constexpr int DT = D / 32;      // 32-row tiles of O^T
+  constexpr int RB = D * 2;       // bytes per tile row
+  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTK, D, NW>() + 1;  // per wave and tile
+  static_assert(STAGES == 3, "the loop below keeps two tiles in flight");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -183,20 +137,26 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
     if (valid) {
       const int64_t mi = (int64_t)b * p.n_qblocks + qrow[qt] / p.qbs;
       col_lo[qt] = p.lower[mi] * p.kbs;
-      col_width[qt] = (unsigned)max(p.upper[mi] * p.kbs - col_lo[qt], 0);
+      // keys at or beyond kv_len are never attendable (their LDS rows hold a copy of the last row)
+      col_width[qt] = (unsigned)max(min(p.upper[mi] * p.kbs, p.kv_len) - col_lo[qt], 0);
     }
     mine[qt] = wave_parts(valid && col_width[qt] > 0, qseg[qt], qpos[qt]);
   }
 
-  // ---- live-tile bitmaps: which kv tiles of [t_lo, t_hi) can this wave's rows interact with --
-  unsigned long long* live = reinterpret_cast<unsigned long long*>(smem + 2 * Smem::kStage);
+  // ---- live tiles: each wave marks the kv tiles of [t_lo, t_hi) its rows can interact with; the
+  // union is compacted into a list the work-group then walks -------------------------------------
+  int* live_count = reinterpret_cast<int*>(smem + Smem::kTotal);
+  unsigned long long* live_bits = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal + 16);
   const int word0 = t_lo >> 6;
   const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
-  const unsigned long long* my_live = live + wave * words;
+  const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.n_kv_tiles, 64) + 1));
   mark_live_tiles<true, MQ>(p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles, mine, t_lo, t_hi,
-                            live + wave * words, word0, lane);
+                            live_bits + wave * words, word0, lane);
   __syncthreads();
-  int t = next_live_tile<NW>(live, words, word0, t_lo - 1);
+  if (wave == 0)
+    compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
+  __syncthreads();
+  const int n_live = *live_count;
 
   f32x16 o[DT][MQ];
   float m_run[MQ], l_run[MQ];
@@ -210,7 +170,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
       for (int i = 0; i < 16; i++) o[dt][qt][i] = 0.f;
   }
 
-  if (t < t_hi) {
+  if (n_live > 0) {
     // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step.
     // A negative scale is folded into Q so that the softmax below can assume scale_log2 > 0.
     vec8 qf[MQ][KSTEPS];
@@ -228,23 +188,51 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
     }
     const float cs = p.scale_log2;  // > 0
 
-    TileLoader<D, NT> loader;
-    loader.load(p, kbase, vbase, kv_seg, kv_pos, t * kTK, tid);
-    loader.store(smem, tid);
-    __syncthreads();
+    // per-lane offsets into a swizzled tile
+    int nat_off[KSTEPS], tr_off[DT][2];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) nat_off[ks] = nat_offset<D>(c, ks, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      tr_off[dt][0] = tr_offset<D>(lane, dt, 0);
+      tr_off[dt][1] = tr_offset<D>(lane, dt, 1);
+    }
 
-    for (int buf = 0; t < t_hi; buf ^= 1) {
-      const int kv0 = t * kTK;
-      char* stage = smem + buf * Smem::kStage;
-      char* next_stage = smem + (buf ^ 1) * Smem::kStage;
-      const int t_next = next_live_tile<NW>(live, words, word0, t);
-      const bool has_next = t_next < t_hi;
-      if (has_next) loader.load(p, kbase, vbase, kv_seg, kv_pos, t_next * kTK, tid);
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
+    const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
+    auto issue = [&](int tile, int stage) {
+      const uint32_t base = smem_addr + stage * Smem::kStage;
+      async_tile_copy<kTK, D, NW>(kbase, p.k_ss * 2, tile * kTK, p.kv_len, base, wave, lane);
+      async_tile_copy<kTK, D, NW>(vbase, p.v_ss * 2, tile * kTK, p.kv_len, base + Smem::kTileBytes, wave, lane);
+      async_copy_b32(id_src + min(tile * kTK + lane, p.kv_len - 1),
+                     __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + (wave & 1) * (kTK * 4)));
+    };
 
-      if (tile_is_live(my_live, word0, t)) {
-        const char* ktile = stage;
-        const char* vtile = stage + Smem::kKBytes;
-        const int32_t* ids = reinterpret_cast<const int32_t*>(stage + Smem::kKBytes + Smem::kVBytes);
+    // entries of the live list for iterations i, i + 1, i + 2 (read ahead of their use)
+    uint32_t e0 = live_list[0];
+    uint32_t e1 = n_live > 1 ? live_list[1] : 0;
+    uint32_t e2 = n_live > 2 ? live_list[2] : 0;
+    issue(e0 & 0xffffff, 0);
+    if (n_live > 1) issue(e1 & 0xffffff, 1);
+
+    int stage = 0;
+    for (int i = 0; i < n_live; i++) {
+      // tile i has landed once at most the copies of tile i + 1 are outstanding
+#ifndef KVAX_EXP_NOBAR
+      if (i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      __syncthreads();
+#endif
+      const uint32_t e3 = i + 3 < n_live ? live_list[i + 3] : 0;
+#ifndef KVAX_EXP_NOCOPY
+      if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+#endif
+      const int t = e0 & 0xffffff;
+
+      if ((e0 >> (24 + wave)) & 1) {
+        const int kv0 = t * kTK;
+        const char* ktile = smem + stage * Smem::kStage;
+        const char* vtile = ktile + Smem::kTileBytes;
+        const int32_t* ids = reinterpret_cast<const int32_t*>(ktile + 2 * Smem::kTileBytes);
 
         // ---- S^T = K Q^T -----------------------------------------------------------------
         f32x16 s[2][MQ];
@@ -259,7 +247,11 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
           vec8 a[2];
 #pragma unroll
           for (int kt = 0; kt < 2; kt++)
-            a[kt] = read_row8<Tr>(ktile, Smem::kKStride, 32 * kt + c, 16 * ks + 8 * h);
+#ifdef KVAX_EXP_NOLDS
+            a[kt] = qf[0][(ks + kt) % KSTEPS];
+#else
+            a[kt] = *reinterpret_cast<const vec8*>(ktile + 32 * kt * RB + nat_off[ks]);
+#endif
 #pragma unroll
           for (int kt = 0; kt < 2; kt++)
 #pragma unroll
@@ -276,8 +268,19 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
                                 col_lo[qt], col_width[qt], -INFINITY);
         }
 
-        // ---- online softmax (per query column = per lane, halves combined once) ------------
         vec8 pb[2][2][MQ];
+#ifdef KVAX_EXP_NOVALU
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+          for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+              f32x4 w = {s[kt][qt][8 * st], s[kt][qt][8 * st + 1], s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3]};
+              pb[kt][st][qt] = __builtin_bit_cast(vec8, w);
+            }
+#else
+        // ---- online softmax (per query column = per lane, halves combined once) ------------
 #pragma unroll
         for (int qt = 0; qt < MQ; qt++) {
           float mx = s[0][qt][0];
@@ -315,6 +318,7 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
           l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
         }
 
+#endif
         // ---- O^T += V^T P^T ---------------------------------------------------------------
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
@@ -322,15 +326,17 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-              const vec8 a = tr_read_a<Tr>(vtile, Smem::kVStride, 32 * kt + 16 * st, 32 * dt, lane);
+#ifdef KVAX_EXP_NOLDS
+              const vec8 a = qf[0][(dt + st + 2 * kt) % KSTEPS];
+#else
+              const vec8 a = tr_read_a_swz<Tr>(vtile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+#endif
 #pragma unroll
               for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
             }
       }
-
-      if (has_next) loader.store(next_stage, tid);
-      __syncthreads();
-      t = t_next;
+      e0 = e1, e1 = e2, e2 = e3;
+      stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
   }
 
@@ -356,16 +362,18 @@ __global__ __launch_bounds__(NW * 64, OCC) void fa_fwd_kernel(const FwdParams p)
   }
 }
 
-template <class Tr, int D, int MQ, int NW, int OCC>
+template <class Tr, int D, int MQ, int NW, int WPS>
 int launch_fwd(const FwdParams& p0, hipStream_t stream) {
+  constexpr int STAGES = 3;
   FwdParams p = p0;
   constexpr int TQ = NW * 32 * MQ;
   p.num_q_tiles = cdiv(p.q_len, TQ);
   p.total_items = p.batch * p.num_heads * p.num_q_tiles;
   if (p.total_items == 0) return KVAX_OK;
-  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, OCC>;
-  const int smem = FwdSmem<D>::kTotal + NW * (cdiv(p.n_kv_tiles, 64) + 1) * 8;
-  constexpr int kMaxSmem = 160 * 1024 / OCC;
+  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES>;
+  const int smem = FwdSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
+  constexpr int kWgPerCu = (WPS * 4 / NW) > 0 ? (WPS * 4 / NW) : 1;
+  constexpr int kMaxSmem = 160 * 1024 / kWgPerCu;
   if (smem > kMaxSmem)
     return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
                 p.kv_len, smem, kMaxSmem);
@@ -461,7 +469,12 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
   const bool bf16 = a->dtype == KVAX_BF16;
+  if (const char* v = getenv("KVAX_FWD_VARIANT")) {  // experiment switch
+    if (a->head_dim == 128 && bf16) {
+      if (v[0] == 'a') return launch_fwd<Bf16, 128, 1, 4, 1>(p, stream);
+    }
+  }
   if (a->head_dim == 128)
-    return bf16 ? launch_fwd<Bf16, 128, 1, 4, 2>(p, stream) : launch_fwd<F16, 128, 1, 4, 2>(p, stream);
-  return bf16 ? launch_fwd<Bf16, 64, 1, 4, 2>(p, stream) : launch_fwd<F16, 64, 1, 4, 2>(p, stream);
+    return bf16 ? launch_fwd<Bf16, 128, 1, 8, 2>(p, stream) : launch_fwd<F16, 128, 1, 8, 2>(p, stream);
+  return bf16 ? launch_fwd<Bf16, 64, 1, 8, 2>(p, stream) : launch_fwd<F16, 64, 1, 8, 2>(p, stream);
 }

@@ -121,6 +121,14 @@ def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd
     return out, lse
 
 
+def backward_workspace_bytes(query, key) -> int:
+    """Size of the scratch buffer ``kvax_fa_bwd`` needs for these shapes (delta + tile summaries)."""
+    a = _native.FaArgs()
+    a.batch, a.q_len, a.num_heads = query.shape[0], query.shape[1], query.shape[2]
+    a.kv_len, a.num_kv_heads, a.head_dim = key.shape[1], key.shape[2], key.shape[3]
+    return int(_native.lib().kvax_fa_bwd_workspace_bytes(C.byref(a)))
+
+
 def flash_attention_backward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, dq_mask, dkdv_mask,
                              out, lse, dout, scale, fwd_params, bwd_params, dkdv_fp32=False,
                              flags=0, buffers=None):
