@@ -60,6 +60,8 @@ struct BwdParams {
   int n_kv_tiles, n_q_tiles;
   int flags;
   float scale, scale_log2;
+  float scale_log2_abs;  // |scale| * log2(e) > 0, used with K negated when the scale is negative
+  uint32_t k_sign;       // 0x80008000 when the scale is negative
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
   constexpr int DT = D / 32;
   constexpr int RB = D * 2;
   constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
-  static_assert(STAGES == 3, "the loop below keeps two tiles in flight");
+  static_assert(STAGES == 4, "two tiles in flight, one being read by the previous unit");
   static_assert(NW >= 4 && NW % 4 == 0, "one wave per row-data array");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -408,6 +410,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
           u = *reinterpret_cast<const uint4*>(kr + (16 * ks + 8 * h) * 2);
           w = *reinterpret_cast<const uint4*>(vr + (16 * ks + 8 * h) * 2);
         }
+        u.x ^= p.k_sign, u.y ^= p.k_sign, u.z ^= p.k_sign, u.w ^= p.k_sign;
         kf[ks] = __builtin_bit_cast(vec8, u);
         vf[ks] = __builtin_bit_cast(vec8, w);
       }
@@ -442,83 +445,139 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
     };
     auto entry_of = [&](int step) { return live_list[step % n_live]; };
 
+    // ---- the phases of one unit = 32 query rows (mt) of one tile ------------------------------
+    // A: S = Q K^T and dP = dO V^T (32 MFMAs); operand reads run two contraction steps ahead
+    auto phase_a = [&](const char* qrows, const char* dorows, f32x16& s, f32x16& dp) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
+      vec8 qa[KSTEPS], da[KSTEPS];
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        qa[ks] = *reinterpret_cast<const vec8*>(qrows + nat_off[ks]);
+        da[ks] = *reinterpret_cast<const vec8*>(dorows + nat_off[ks]);
+      }
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        if (ks + 2 < KSTEPS) {
+          qa[ks + 2] = *reinterpret_cast<const vec8*>(qrows + nat_off[ks + 2]);
+          da[ks + 2] = *reinterpret_cast<const vec8*>(dorows + nat_off[ks + 2]);
+        }
+        s = Tr::mfma(qa[ks], kf[ks], s);
+        dp = Tr::mfma(da[ks], vf[ks], dp);
+      }
+      // issue order: 4 reads ahead, then one read per MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * KSTEPS - 4; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    };
+    // B + C in one basic block: P = exp2(S * |c| - lse), dS = P * (dP - delta), both rounded to the
+    // input dtype, for the current unit -- together with dV^T += dO^T P, dK^T += Q^T dS of the
+    // previous unit (32 MFMAs fed by transposing reads), so that the exponentials and
+    // conversions issue in the shadow of the MFMAs.
+    auto phase_bc = [&](const float* rows, f32x16& s, f32x16& dp, vec8 (&pb)[2], vec8 (&dsb)[2],
+                        const char* qprev, const char* doprev, const vec8 (&pbp)[2], const vec8 (&dsbp)[2]) {
+      float ls[16], dl[16];
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const float4 lse4 = *reinterpret_cast<const float4*>(rows + 8 * g4 + 4 * h);
+        const float4 del4 = *reinterpret_cast<const float4*>(rows + kTile + 8 * g4 + 4 * h);
+        ls[4 * g4] = lse4.x, ls[4 * g4 + 1] = lse4.y, ls[4 * g4 + 2] = lse4.z, ls[4 * g4 + 3] = lse4.w;
+        dl[4 * g4] = del4.x, dl[4 * g4 + 1] = del4.y, dl[4 * g4 + 2] = del4.z, dl[4 * g4 + 3] = del4.w;
+      }
+#pragma unroll
+      for (int st = 0; st < 2; st++) {
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+          const vec8 ad = tr_read_a_swz<Tr>(doprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
+          const vec8 aq = tr_read_a_swz<Tr>(qprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
+          dv[dt] = Tr::mfma(ad, pbp[st], dv[dt]);
+          dk[dt] = Tr::mfma(aq, dsbp[st], dk[dt]);
+          // a quarter of the unit's element-wise work per pair of MFMAs
+          const int i0 = 8 * st + dt * (8 / DT);
+#pragma unroll
+          for (int i = i0; i < i0 + 8 / DT; i++) {
+            s[i] = fast_exp2(__builtin_fmaf(s[i], p.scale_log2_abs, -ls[i]));
+            dp[i] = s[i] * (dp[i] - dl[i]);
+          }
+        }
+        pb[st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                           s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+        dsb[st] = pack8<Tr>(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
+                            dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
+      }
+    };
+    // C alone (after the last unit)
+    auto phase_c = [&](const char* qprev, const char* doprev, const vec8 (&pbp)[2], const vec8 (&dsbp)[2]) {
+#pragma unroll
+      for (int st = 0; st < 2; st++)
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+          const vec8 ad = tr_read_a_swz<Tr>(doprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
+          const vec8 aq = tr_read_a_swz<Tr>(qprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
+          dv[dt] = Tr::mfma(ad, pbp[st], dv[dt]);
+          dk[dt] = Tr::mfma(aq, dsbp[st], dk[dt]);
+        }
+    };
+
     uint32_t e0 = entry_of(0);
     uint32_t e1 = steps > 1 ? entry_of(1) : 0;
     uint32_t e2 = steps > 2 ? entry_of(2) : 0;
     issue(0, e0, 0);
     if (steps > 1) issue(1, e1, 1);
 
+    // Software pipeline over units: phase C of the previous unit is issued together with phase B
+    // of the current one.  A unit the wave has no part in contributes zero operands; before the
+    // first unit the "previous" operands are zero and point at the first tile, which has landed.
+    vec8 pb_prev[2], dsb_prev[2];
+    const vec8 zero8 = __builtin_bit_cast(vec8, make_uint4(0, 0, 0, 0));
+    pb_prev[0] = pb_prev[1] = dsb_prev[0] = dsb_prev[1] = zero8;
+    const char* q_prev = smem;
+    const char* do_prev = smem + Smem::kTileBytes;
+
     int stage = 0;
     for (int step = 0; step < steps; step++) {
       if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
       const uint32_t e3 = step + 3 < steps ? entry_of(step + 3) : 0;
-      if (step + 2 < steps) issue(step + 2, e2, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      if (step + 2 < steps) issue(step + 2, e2, (stage + 2) % STAGES);
       const int t = e0 & 0xffffff;
+      const bool active = (e0 >> (24 + wave)) & 1;
+      const int qr0 = t * kTile;
+      const char* qtile = smem + stage * Smem::kStage;
+      const char* dotile = qtile + Smem::kTileBytes;
+      const float* rowdata = reinterpret_cast<const float*>(qtile + 2 * Smem::kTileBytes);
+      const int32_t* rowids = reinterpret_cast<const int32_t*>(rowdata + 2 * kTile);
+      const bool full = t >= tf_lo && t < tf_hi;
 
-      if ((e0 >> (24 + wave)) & 1) {
-        const int qr0 = t * kTile;
-        const char* qtile = smem + stage * Smem::kStage;
-        const char* dotile = qtile + Smem::kTileBytes;
-        const float* rowdata = reinterpret_cast<const float*>(qtile + 2 * Smem::kTileBytes);
-        const int32_t* rowids = reinterpret_cast<const int32_t*>(rowdata + 2 * kTile);
-        const bool full = t >= tf_lo && t < tf_hi;
-
+      if (!active) {
+        // nothing of this tile concerns the wave: retire the pending unit and carry zero operands
+        phase_c(q_prev, do_prev, pb_prev, dsb_prev);
+        pb_prev[0] = pb_prev[1] = dsb_prev[0] = dsb_prev[1] = zero8;
+        q_prev = qtile;
+        do_prev = dotile;
+      } else {
 #pragma unroll
         for (int mt = 0; mt < 2; mt++) {
           f32x16 s, dp;
-#pragma unroll
-          for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
-#pragma unroll
-          for (int ks = 0; ks < KSTEPS; ks++) {
-            const vec8 qa = *reinterpret_cast<const vec8*>(qtile + 32 * mt * RB + nat_off[ks]);
-            const vec8 da = *reinterpret_cast<const vec8*>(dotile + 32 * mt * RB + nat_off[ks]);
-            s = Tr::mfma(qa, kf[ks], s);
-            dp = Tr::mfma(da, vf[ks], dp);
-          }
-#pragma unroll
-          for (int g4 = 0; g4 < 4; g4++) {
-            const int r0 = 32 * mt + 8 * g4 + 4 * h;
-            const float4 lse4 = *reinterpret_cast<const float4*>(rowdata + r0);
-            const float ls[4] = {lse4.x, lse4.y, lse4.z, lse4.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-              s[4 * g4 + j] = fast_exp2(__builtin_fmaf(s[4 * g4 + j], p.scale_log2, -ls[j]));
-          }
-          if (!full)
+          phase_a(qtile + 32 * mt * RB, dotile + 32 * mt * RB, s, dp);
+          if (!full)  // raw scores: masked -> -inf, so that P = exp2(-inf) = 0 (scale_log2_abs > 0)
             mask_c_tile<false>(s, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
-                               col_width, 0.f);
-#pragma unroll
-          for (int g4 = 0; g4 < 4; g4++) {
-            const int r0 = 32 * mt + 8 * g4 + 4 * h;
-            const float4 del4 = *reinterpret_cast<const float4*>(rowdata + kTile + r0);
-            const float dl[4] = {del4.x, del4.y, del4.z, del4.w};
-#pragma unroll
-            for (int j = 0; j < 4; j++) dp[4 * g4 + j] = s[4 * g4 + j] * (dp[4 * g4 + j] - dl[j]);
-          }
+                               col_width, -INFINITY);
           vec8 pb[2], dsb[2];
-#pragma unroll
-          for (int st = 0; st < 2; st++) {
-            pb[st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
-                               s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
-            dsb[st] = pack8<Tr>(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
-                                dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
-          }
-          // dV^T += dO^T P ; dK^T += Q^T dS
-#pragma unroll
-          for (int st = 0; st < 2; st++)
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-              const vec8 ad = tr_read_a_swz<Tr>(dotile + (32 * mt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
-              dv[dt] = Tr::mfma(ad, pb[st], dv[dt]);
-              const vec8 aq = tr_read_a_swz<Tr>(qtile + (32 * mt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
-              dk[dt] = Tr::mfma(aq, dsb[st], dk[dt]);
-            }
+          phase_bc(rowdata + 32 * mt, s, dp, pb, dsb, q_prev, do_prev, pb_prev, dsb_prev);
+          pb_prev[0] = pb[0], pb_prev[1] = pb[1], dsb_prev[0] = dsb[0], dsb_prev[1] = dsb[1];
+          q_prev = qtile + 32 * mt * RB;
+          do_prev = dotile + 32 * mt * RB;
         }
       }
       e0 = e1, e1 = e2, e2 = e3;
       stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
+    phase_c(q_prev, do_prev, pb_prev, dsb_prev);
   }
 
   if (in && p.dkdv_f32) {
@@ -599,9 +658,9 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   // dK/dV: 4 wavefronts (128 kv rows) per work-group, one per SIMD
   if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
     constexpr int NW = 4;
-    auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW, 1, STAGES>;
+    auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW, 1, 4>;
     static bool done = false;
-    const int smem = DkdvSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
+    const int smem = DkdvSmem<D, 4>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
     if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, NW * 32);
     p.total_items = p.batch * p.num_kv_heads * p.num_tiles;
@@ -677,6 +736,8 @@ extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.flags = a->flags;
   p.scale = a->scale;
   p.scale_log2 = a->scale * 1.4426950408889634f;
+  p.scale_log2_abs = fmaxf(fabsf(a->scale), 1e-30f) * 1.4426950408889634f;
+  p.k_sign = a->scale < 0.f ? 0x80008000u : 0u;
   hipStream_t stream = (hipStream_t)stream_;
   const bool bf16 = a->dtype == KVAX_BF16;
   if (a->head_dim == 128)
