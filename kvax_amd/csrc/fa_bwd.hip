@@ -147,13 +147,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   const int wave = tid / 64, lane = tid % 64;
   const int c = lane % 32, h = lane / 32;
 
-  int item = xcd_contiguous(blockIdx.x, p.total_items);
-  const int g = item % p.group;
-  item /= p.group;
-  const int q_tile = p.num_tiles - 1 - item % p.num_tiles;
-  item /= p.num_tiles;
-  const int kv_head = item % p.num_kv_heads;
-  const int b = item / p.num_kv_heads;
+  int group, rank, g;
+  const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, p.group};
+  if (!items.decode(blockIdx.x, group, rank, g)) return;
+  const int q_tile = p.num_tiles - 1 - rank;
+  const int kv_head = group % p.num_kv_heads;
+  const int b = group / p.num_kv_heads;
   const int head = kv_head * p.group + g;
   const int q0 = q_tile * TQ;
 
@@ -234,10 +233,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
     const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
+    const AsyncTileCopy<kTile, D, NW> copy_k(p.k_ss * 2, wave, lane), copy_v(p.v_ss * 2, wave, lane);
     auto issue = [&](int tile, int stage) {
       const uint32_t base = smem_addr + stage * Smem::kStage;
-      async_tile_copy<kTile, D, NW>(kbase, p.k_ss * 2, tile * kTile, p.kv_len, base, wave, lane);
-      async_tile_copy<kTile, D, NW>(vbase, p.v_ss * 2, tile * kTile, p.kv_len, base + Smem::kTileBytes, wave, lane);
+      copy_k(kbase, tile * kTile, p.kv_len, base);
+      copy_v(vbase, tile * kTile, p.kv_len, base + Smem::kTileBytes);
       async_copy_b32(id_src + min(tile * kTile + lane, p.kv_len - 1),
                      __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + (wave & 1) * (kTile * 4)));
     };
@@ -347,11 +347,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
   const int c = lane % 32, h = lane / 32;
 
   // early kv tiles see the most queries under a causal mask: run them first
-  int item = xcd_contiguous(blockIdx.x, p.total_items);
-  const int kv_tile = item % p.num_tiles;
-  item /= p.num_tiles;
-  const int kv_head = item % p.num_kv_heads;
-  const int b = item / p.num_kv_heads;
+  int group, kv_tile, member;
+  const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, 1};
+  if (!items.decode(blockIdx.x, group, kv_tile, member)) return;
+  const int kv_head = group % p.num_kv_heads;
+  const int b = group / p.num_kv_heads;
   const int k0 = kv_tile * TKV;
 
   const int kbs = p.bk, qbs = p.bq;
@@ -426,15 +426,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
     const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos
+    const AsyncTileCopy<kTile, D, NW> copy_q(p.q_ss * 2, wave, lane), copy_do(p.do_ss * 2, wave, lane);
     // step s = (head s / n_live of the group, list entry s % n_live)
     auto issue = [&](int step, uint32_t entry, int stage) {
       const int head = kv_head * p.group + step / n_live;
       const int qr0 = (int)(entry & 0xffffff) * kTile;
       const uint32_t base = smem_addr + stage * Smem::kStage;
-      async_tile_copy<kTile, D, NW>(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, p.q_ss * 2, qr0,
-                                    p.q_len, base, wave, lane);
-      async_tile_copy<kTile, D, NW>(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, p.do_ss * 2,
-                                    qr0, p.q_len, base + Smem::kTileBytes, wave, lane);
+      copy_q(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, qr0, p.q_len, base);
+      copy_do(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, qr0, p.q_len, base + Smem::kTileBytes);
       const int qi = min(qr0 + lane, p.q_len - 1);
       const int64_t hoff = ((int64_t)b * p.num_heads + head) * p.q_len + qi;
       const int64_t boff = (int64_t)b * p.q_len + qi;
@@ -651,7 +650,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
     if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dQ kernel")) return rc;
     p.num_tiles = cdiv(p.q_len, NW * 32);
-    p.total_items = p.batch * p.num_heads * p.num_tiles;
+    p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, p.group}.grid();
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
   }
@@ -663,7 +662,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     const int smem = DkdvSmem<D, 4>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
     if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, NW * 32);
-    p.total_items = p.batch * p.num_kv_heads * p.num_tiles;
+    p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, 1}.grid();
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dkdv_kernel")) return rc;
   }

@@ -113,14 +113,48 @@ __device__ __forceinline__ int cdiv_dev(int a, int b) { return (a + b - 1) / b; 
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32); }
 
-// Work-group index -> work item, so that each XCD (work-groups are dealt round-robin to the 8
-// XCDs) walks a contiguous range of items and neighbouring items share that XCD's L2.
-__device__ __forceinline__ int xcd_contiguous(int linear, int total) {
-  constexpr int kXcds = 8;
-  const int per = total / kXcds, rem = total % kXcds;
-  const int xcd = linear % kXcds, idx = linear / kXcds;
-  return xcd * per + (xcd < rem ? xcd : rem) + idx;
-}
+// Work distribution.  Work-groups are dealt round-robin to the 8 XCDs (work-group L runs on XCD
+// L % 8, each XCD has its own L2), so the map from L to a work item decides both L2 sharing and
+// balance.  Items are (group, tile rank, member): a group is one (batch, kv head) -- everything
+// that reads the same K/V -- with `tiles` tiles ranked heaviest first and `members` query heads
+// per tile.  With at least 8 groups each XCD owns whole groups; with fewer (and 8 divisible by
+// the count) the tiles of a group are dealt round-robin to the XCDs that share it, so that every
+// XCD gets the same mix of heavy and light tiles; otherwise items are cut into 8 contiguous runs.
+struct ItemMap {
+  int groups, tiles, members;
+  __host__ __device__ int mode() const { return groups >= 8 ? 0 : (8 % groups == 0 ? 1 : 2); }
+  __host__ __device__ int grid() const {
+    if (mode() == 0) return 8 * members * ((groups + 7) / 8) * tiles;
+    if (mode() == 1) return 8 * members * ((tiles + 8 / groups - 1) / (8 / groups));
+    return groups * tiles * members;
+  }
+  // false when work-group L has nothing to do
+  __device__ __forceinline__ bool decode(int L, int& group, int& rank, int& member) const {
+    const int x = L % 8, j = L / 8;
+    if (mode() == 0) {
+      const int per_xcd = (groups + 7) / 8;
+      member = j % members;
+      group = x + 8 * ((j / members) % per_xcd);
+      rank = j / (members * per_xcd);
+      return group < groups && rank < tiles;
+    }
+    if (mode() == 1) {
+      const int share = 8 / groups;
+      member = j % members;
+      group = x / share;
+      rank = x % share + share * (j / members);
+      return rank < tiles;
+    }
+    const int total = groups * tiles * members;
+    const int per = total / 8, rem = total % 8;
+    int item = x * per + (x < rem ? x : rem) + j;
+    member = item % members;
+    item /= members;
+    rank = item % tiles;
+    group = item / tiles;
+    return true;
+  }
+};
 
 
 // ---------------------------------------------------------------------------------------------
@@ -309,28 +343,59 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
+// Same with a wave-uniform 64-bit base address (held in SGPRs) plus a 32-bit per-lane byte offset:
+// no vector ALU work per copy.
+__device__ __forceinline__ void async_copy_b128(const char* sbase, uint32_t lane_off, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(lane_off),
+               "s"(sbase)
+               : "memory");
+}
+
 // Copies rows [row0, row0 + ROWS) of a row-major global matrix (16-bit elements, D per row,
 // `row_stride_bytes` between rows) into a swizzled LDS tile at LDS address `tile_addr`.  Rows at
 // or beyond `limit` (>= 1) are replaced by row limit - 1: callers mask them out by index.
-// Every wave issues ROWS * D * 2 / 1024 / NW copies.
+// Every wave issues ROWS * D * 2 / 1024 / NW copies; the per-lane part of the source address is
+// computed once (in the constructor) and only a scalar base changes from tile to tile.
 template <int ROWS, int D, int NW>
-__device__ __forceinline__ void async_tile_copy(const char* gbase, int64_t row_stride_bytes, int row0,
-                                                int limit, uint32_t tile_addr, int wave, int lane) {
-  constexpr int kRowsPerCopy = 1024 / (D * 2);  // 4 (D = 128) or 8 (D = 64)
-  constexpr int kCopies = ROWS / kRowsPerCopy;
-  constexpr int kChunks = D / 8;
+struct AsyncTileCopy {
+  static constexpr int kRowsPerCopy = 1024 / (D * 2);  // 4 (D = 128) or 8 (D = 64)
+  static constexpr int kCopies = ROWS / kRowsPerCopy;
+  static constexpr int kPerWave = kCopies / NW;
+  static constexpr int kChunks = D / 8;
   static_assert(kCopies % NW == 0, "copies must split evenly over the waves");
-  const int rin = lane / kChunks, pos = lane % kChunks;
+  uint32_t lane_off[kPerWave];  // rin * stride + chunk * 16 for each of the wave's copies
+  int64_t stride;
+  int wave_u, rin, pos;
+
+  __device__ __forceinline__ AsyncTileCopy(int64_t row_stride_bytes, int wave, int lane)
+      : stride(row_stride_bytes), wave_u(__builtin_amdgcn_readfirstlane(wave)), rin(lane / kChunks),
+        pos(lane % kChunks) {
 #pragma unroll
-  for (int j = 0; j < kCopies / NW; j++) {
-    const int grp = j * NW + wave;
-    const int r = grp * kRowsPerCopy + rin;
-    const int chunk = pos ^ swz<D>(r);
-    const int grow = min(row0 + r, limit - 1);
-    async_copy_b128(gbase + (int64_t)grow * row_stride_bytes + chunk * 16,
-                    __builtin_amdgcn_readfirstlane(tile_addr + grp * 1024));
+    for (int j = 0; j < kPerWave; j++) {
+      const int r = (j * NW + wave_u) * kRowsPerCopy + rin;
+      lane_off[j] = (uint32_t)(rin * row_stride_bytes) + (uint32_t)((pos ^ swz<D>(r)) * 16);
+    }
   }
-}
+
+  __device__ __forceinline__ void operator()(const char* gbase, int row0, int limit, uint32_t tile_addr) const {
+    if (row0 + ROWS <= limit) {  // whole tile in range (uniform): scalar base + fixed lane offsets
+#pragma unroll
+      for (int j = 0; j < kPerWave; j++) {
+        const int grp = j * NW + wave_u;
+        async_copy_b128(gbase + (int64_t)(row0 + grp * kRowsPerCopy) * stride, lane_off[j],
+                        tile_addr + grp * 1024);
+      }
+    } else {  // ragged tail: clamp each lane's row
+#pragma unroll
+      for (int j = 0; j < kPerWave; j++) {
+        const int grp = j * NW + wave_u;
+        const int r = grp * kRowsPerCopy + rin;
+        const int grow = min(row0 + r, limit - 1);
+        async_copy_b128(gbase + (int64_t)grow * stride + (pos ^ swz<D>(r)) * 16, tile_addr + grp * 1024);
+      }
+    }
+  }
+};
 template <int ROWS, int D, int NW>
 constexpr int async_tile_copies_per_wave() {
   return ROWS / (1024 / (D * 2)) / NW;

@@ -11,12 +11,12 @@
 // query column of the 32x32 MFMA result.  Row max / row sum are then in-lane reductions plus a
 // single exchange between the two half-waves, and the exponentiated tile is already in the
 // B-operand layout of the second contraction O^T += V^T P^T -- P never goes through LDS.  V^T
-// operands are gathered from the row-major V tile with transposing LDS reads.  K/V tiles are
-// staged through LDS once per work-group (double buffered, prefetched through registers) and
-// shared by the work-group's wavefronts; the query heads of one GQA group run as neighbouring
-// work-groups on one XCD so K/V tiles are served from that XCD's L2.
-#include <cstdlib>
-
+// operands are gathered from the row-major V tile with transposing LDS reads.  K/V tiles reach
+// LDS by asynchronous global->LDS copies (no registers involved) into a ring of swizzled stages,
+// two tiles ahead of the one being consumed, and are shared by the work-group's 8 wavefronts
+// (256 query rows); the query heads of one GQA group run as neighbouring work-groups on one XCD
+// so K/V tiles are served from that XCD's L2.  Tiles of the block-mask range in which no
+// (query, key) pair can pass the element mask are dropped up front (fa_tiles.hip).
 #include "common.h"
 #include "fa_common.h"
 
@@ -79,13 +79,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   const int c = lane % 32, h = lane / 32;
 
   // ---- work item: heads of a GQA group adjacent, long (late) query tiles first -------------
-  int item = xcd_contiguous(blockIdx.x, p.total_items);
-  const int g = item % p.group;
-  item /= p.group;
-  const int q_tile = p.num_q_tiles - 1 - item % p.num_q_tiles;
-  item /= p.num_q_tiles;
-  const int kv_head = item % p.num_kv_heads;
-  const int b = item / p.num_kv_heads;
+  int group, rank, g;
+  const ItemMap items{p.batch * p.num_kv_heads, p.num_q_tiles, p.group};
+  if (!items.decode(blockIdx.x, group, rank, g)) return;
+  const int q_tile = p.num_q_tiles - 1 - rank;
+  const int kv_head = group % p.num_kv_heads;
+  const int b = group / p.num_kv_heads;
   const int head = kv_head * p.group + g;
   const int q0 = q_tile * TQ;
 
@@ -200,10 +199,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
     const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
+    const AsyncTileCopy<kTK, D, NW> copy_k(p.k_ss * 2, wave, lane), copy_v(p.v_ss * 2, wave, lane);
     auto issue = [&](int tile, int stage) {
       const uint32_t base = smem_addr + stage * Smem::kStage;
-      async_tile_copy<kTK, D, NW>(kbase, p.k_ss * 2, tile * kTK, p.kv_len, base, wave, lane);
-      async_tile_copy<kTK, D, NW>(vbase, p.v_ss * 2, tile * kTK, p.kv_len, base + Smem::kTileBytes, wave, lane);
+      copy_k(kbase, tile * kTK, p.kv_len, base);
+      copy_v(vbase, tile * kTK, p.kv_len, base + Smem::kTileBytes);
       async_copy_b32(id_src + min(tile * kTK + lane, p.kv_len - 1),
                      __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + (wave & 1) * (kTK * 4)));
     };
@@ -218,14 +218,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     int stage = 0;
     for (int i = 0; i < n_live; i++) {
       // tile i has landed once at most the copies of tile i + 1 are outstanding
-#ifndef KVAX_EXP_NOBAR
       if (i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
-#endif
       const uint32_t e3 = i + 3 < n_live ? live_list[i + 3] : 0;
-#ifndef KVAX_EXP_NOCOPY
       if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
-#endif
       const int t = e0 & 0xffffff;
 
       if ((e0 >> (24 + wave)) & 1) {
@@ -247,16 +243,20 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           vec8 a[2];
 #pragma unroll
           for (int kt = 0; kt < 2; kt++)
-#ifdef KVAX_EXP_NOLDS
-            a[kt] = qf[0][(ks + kt) % KSTEPS];
-#else
             a[kt] = *reinterpret_cast<const vec8*>(ktile + 32 * kt * RB + nat_off[ks]);
-#endif
 #pragma unroll
           for (int kt = 0; kt < 2; kt++)
 #pragma unroll
             for (int qt = 0; qt < MQ; qt++) s[kt][qt] = Tr::mfma(a[kt], qf[qt][ks], s[kt][qt]);
         }
+        // issue order: operand reads run four ahead of the MFMAs that consume them
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * KSTEPS - 4; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, MQ, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4 * MQ, 0);
 
         // ---- element mask outside the full range (raw scores; masked -> -inf) -------------
         if (!(t >= tf_lo && t < tf_hi)) {
@@ -269,17 +269,6 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
         }
 
         vec8 pb[2][2][MQ];
-#ifdef KVAX_EXP_NOVALU
-#pragma unroll
-        for (int qt = 0; qt < MQ; qt++)
-#pragma unroll
-          for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-            for (int st = 0; st < 2; st++) {
-              f32x4 w = {s[kt][qt][8 * st], s[kt][qt][8 * st + 1], s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3]};
-              pb[kt][st][qt] = __builtin_bit_cast(vec8, w);
-            }
-#else
         // ---- online softmax (per query column = per lane, halves combined once) ------------
 #pragma unroll
         for (int qt = 0; qt < MQ; qt++) {
@@ -318,7 +307,6 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
         }
 
-#endif
         // ---- O^T += V^T P^T ---------------------------------------------------------------
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
@@ -326,11 +314,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
-#ifdef KVAX_EXP_NOLDS
-              const vec8 a = qf[0][(dt + st + 2 * kt) % KSTEPS];
-#else
               const vec8 a = tr_read_a_swz<Tr>(vtile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
-#endif
 #pragma unroll
               for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
             }
@@ -368,8 +352,8 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   FwdParams p = p0;
   constexpr int TQ = NW * 32 * MQ;
   p.num_q_tiles = cdiv(p.q_len, TQ);
-  p.total_items = p.batch * p.num_heads * p.num_q_tiles;
-  if (p.total_items == 0) return KVAX_OK;
+  p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_q_tiles, p.group}.grid();
+  if (p.batch * p.num_heads * p.num_q_tiles == 0) return KVAX_OK;
   auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES>;
   const int smem = FwdSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   constexpr int kWgPerCu = (WPS * 4 / NW) > 0 ? (WPS * 4 / NW) : 1;
@@ -469,11 +453,6 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
   const bool bf16 = a->dtype == KVAX_BF16;
-  if (const char* v = getenv("KVAX_FWD_VARIANT")) {  // experiment switch
-    if (a->head_dim == 128 && bf16) {
-      if (v[0] == 'a') return launch_fwd<Bf16, 128, 1, 4, 1>(p, stream);
-    }
-  }
   if (a->head_dim == 128)
     return bf16 ? launch_fwd<Bf16, 128, 1, 8, 2>(p, stream) : launch_fwd<F16, 128, 1, 8, 2>(p, stream);
   return bf16 ? launch_fwd<Bf16, 64, 1, 8, 2>(p, stream) : launch_fwd<F16, 64, 1, 8, 2>(p, stream);
