@@ -22,6 +22,23 @@ import numpy as np
 import torch
 
 MFMA_BF16_DENSE_PEAK_TFLOPS = 2516.6  # MI355X datasheet: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+CALIBRATION_BYTES = 1 << 30            # bytes read (and bytes written) by the --pmc-calibration kernel
+ROOT = os.path.dirname(os.path.abspath(__file__))
+
+
+def recorded_traffic(kernel: str, workload_name: str):
+    """HBM bytes per launch of `kernel`, as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and
+    written down in profiles/<kernel>_<workload>_pmc.md (line ``traffic_bytes_per_launch: N``).
+    Hardware counters cannot be read from inside this process; None when no such record exists."""
+    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload_name}_pmc.md")
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1])
+    except OSError:
+        pass
+    return None
 
 WORKLOAD_TEXT = {
     "dense_causal": "dense_causal: B1 S8192 Hq32/Hkv8 D128 bf16, one causal document, block 128, forward only",
@@ -44,6 +61,10 @@ def parse():
     ap.add_argument("--block", type=int, default=128)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run a plain streaming kernel of known size (reads and writes "
+                         f"{CALIBRATION_BYTES >> 20} MiB) so that a rocprofv3 --pmc run of this command "
+                         "shows what FETCH_SIZE / WRITE_SIZE read for a known amount of HBM traffic")
     ap.add_argument("--global-positions", action="store_true",
                     help="positions = token index instead of restarting per document")
     return ap.parse_args()
@@ -156,6 +177,14 @@ def main():
             if events is not None:
                 events[i][1].record()
 
+    if args.pmc_calibration:
+        src = torch.ones(CALIBRATION_BYTES // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            torch.mul(src, 1.0, out=dst)  # elementwise kernel: reads and writes CALIBRATION_BYTES
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -210,7 +239,7 @@ def main():
             "peak": MFMA_BF16_DENSE_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": recorded_traffic(dominant, args.workload),
         },
         "step_frac_of_mfma_peak": value / MFMA_BF16_DENSE_PEAK_TFLOPS,
         "fwd_tflops": f_fwd / (kernel_ms["fa_fwd_kernel"] * 1e-3) / 1e12,

@@ -38,11 +38,6 @@ struct Bf16 {
   __device__ static __forceinline__ float to_float(uint16_t bits) {
     return __builtin_bit_cast(float, (uint32_t)bits << 16);
   }
-  // acc + lo + hi of a packed pair, one instruction (v_dot2c_f32_bf16 with a vector of ones)
-  __device__ static __forceinline__ float add_pair(uint32_t packed, float acc) {
-    const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
-  }
 };
 
 struct F16 {
@@ -56,10 +51,6 @@ struct F16 {
   }
   __device__ static __forceinline__ float to_float(uint16_t bits) {
     return (float)__builtin_bit_cast(_Float16, bits);
-  }
-  __device__ static __forceinline__ float add_pair(uint32_t packed, float acc) {
-    const f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, packed), ones, acc, false);
   }
 };
 

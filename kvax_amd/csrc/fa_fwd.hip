@@ -48,7 +48,8 @@ struct FwdParams {
   int num_q_tiles, total_items;
   const int4* kv_tiles;  // tile summaries [batch, n_kv_tiles]
   int n_kv_tiles;
-  float scale_log2;      // scale * log2(e), folded into Q on load
+  uint32_t q_sign;       // 0x80008000 when the scale is negative: Q is negated on load
+  float scale_log2;      // |scale| * log2(e), > 0
 };
 
 template <int D, int STAGES>
@@ -156,20 +157,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   __syncthreads();
   const int n_live = *live_count;
 
-  // Softmax state per query column.  Scores leave the MFMA already in the log2 domain and relative
-  // to a reference maximum m_ref: Q is pre-multiplied by scale * log2(e) and the accumulator of
-  // S^T = K Q^T starts from -m_ref (neg_ref, the same value in all 16 registers).  m_ref follows the
-  // running maximum lazily: it is moved (and O, l rescaled) only when a score exceeds it by more
-  // than kSlack, so that the common path costs one exp2 per score and no subtraction.
-  constexpr float kSlack = 8.f;  // probabilities stay below 2^8
-  f32x16 o[DT][MQ], neg_ref[MQ];
-  float m_ref[MQ], l_run[MQ];
+  f32x16 o[DT][MQ];
+  float m_run[MQ], l_run[MQ];
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
-    m_ref[qt] = -INFINITY;  // no finite score seen yet
+    m_run[qt] = -1e30f;
     l_run[qt] = 0.f;
-#pragma unroll
-    for (int i = 0; i < 16; i++) neg_ref[qt][i] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -177,8 +170,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   }
 
   if (n_live > 0) {
-    // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step,
-    // pre-multiplied by scale * log2(e) (one extra rounding of Q, below that of the probabilities).
+    // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step.
+    // A negative scale is folded into Q so that the softmax below can assume scale_log2 > 0.
     vec8 qf[MQ][KSTEPS];
 #pragma unroll
     for (int qt = 0; qt < MQ; qt++) {
@@ -188,14 +181,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       for (int ks = 0; ks < KSTEPS; ks++) {
         uint4 u = make_uint4(0, 0, 0, 0);
         if (in) u = *reinterpret_cast<const uint4*>(row + (16 * ks + 8 * h) * 2);
-        const uint32_t w[4] = {u.x, u.y, u.z, u.w};
-        uint32_t r[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-          r[j] = Tr::pack2(Tr::to_float(w[j] & 0xffff) * p.scale_log2, Tr::to_float(w[j] >> 16) * p.scale_log2);
-        qf[qt][ks] = __builtin_bit_cast(vec8, make_uint4(r[0], r[1], r[2], r[3]));
+        u.x ^= p.q_sign, u.y ^= p.q_sign, u.z ^= p.q_sign, u.w ^= p.q_sign;
+        qf[qt][ks] = __builtin_bit_cast(vec8, u);
       }
     }
+    const float cs = p.scale_log2;  // > 0
 
     // per-lane offsets into a swizzled tile
     int nat_off[KSTEPS], tr_off[DT][2];
@@ -245,7 +235,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 #pragma unroll
         for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-          for (int qt = 0; qt < MQ; qt++) s[kt][qt] = neg_ref[qt];
+          for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[kt][qt][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++) {
           vec8 a[2];
@@ -286,38 +278,32 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
           mx = fmaxf(mx, xor32(mx));
-          const bool unset = m_ref[qt] == -INFINITY;
-          const bool move = mx > kSlack || (unset && mx > -INFINITY);
-          if (__any(move)) {  // rare after the first tiles: re-centre the columns that need it
-            const float delta = move ? mx : 0.f;
-            const float alpha = unset ? 1.f : fast_exp2(-delta);  // O and l are still zero when unset
-            if (move) m_ref[qt] = unset ? mx : m_ref[qt] + mx;
-            const float nr = m_ref[qt] == -INFINITY ? 0.f : -m_ref[qt];
+          const float m_new = fmaxf(m_run[qt], mx * cs);
+          if (__any(m_new > m_run[qt])) {
+            const float alpha = fast_exp2(m_run[qt] - m_new);
             l_run[qt] *= alpha;
-#pragma unroll
-            for (int i = 0; i < 16; i++) neg_ref[qt][i] = nr;
-#pragma unroll
-            for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-              for (int i = 0; i < 16; i++) s[kt][qt][i] -= delta;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
               for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
           }
+          m_run[qt] = m_new;
           float sum = 0.f;
 #pragma unroll
-          for (int kt = 0; kt < 2; kt++)
+          for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
-            for (int st = 0; st < 2; st++) {
-              uint32_t w[4];
-#pragma unroll
-              for (int j = 0; j < 4; j++) {
-                w[j] = Tr::pack2(fast_exp2(s[kt][qt][8 * st + 2 * j]), fast_exp2(s[kt][qt][8 * st + 2 * j + 1]));
-                sum = Tr::add_pair(w[j], sum);  // the rounded probabilities, as the MFMA below sees them
-              }
-              pb[kt][st][qt] = __builtin_bit_cast(vec8, make_uint4(w[0], w[1], w[2], w[3]));
+            for (int i = 0; i < 16; i++) {
+              const float e = fast_exp2(__builtin_fmaf(s[kt][qt][i], cs, -m_new));
+              s[kt][qt][i] = e;
+              sum += e;
             }
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+              pb[kt][st][qt] = pack8<Tr>(s[kt][qt][8 * st + 0], s[kt][qt][8 * st + 1],
+                                         s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3],
+                                         s[kt][qt][8 * st + 4], s[kt][qt][8 * st + 5],
+                                         s[kt][qt][8 * st + 6], s[kt][qt][8 * st + 7]);
+          }
           l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
         }
 
@@ -355,7 +341,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           u.y = Tr::pack2(o[dt][qt][4 * g4 + 2] * inv, o[dt][qt][4 * g4 + 3] * inv);
           *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
         }
-      if (h == 0) lse[qrow[qt]] = alive ? m_ref[qt] + fast_log2(l) : 0.f;
+      if (h == 0) lse[qrow[qt]] = alive ? m_run[qt] + fast_log2(l) : 0.f;
     }
   }
 }
@@ -456,7 +442,8 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.group = a->num_heads / a->num_kv_heads;
   p.qbs = a->fwd_query_block, p.kbs = a->fwd_kv_block;
   p.n_qblocks = cdiv(a->q_len, a->fwd_query_block);
-  p.scale_log2 = a->scale * 1.4426950408889634f;
+  p.q_sign = a->scale < 0.f ? 0x80008000u : 0u;
+  p.scale_log2 = fmaxf(fabsf(a->scale), 1e-30f) * 1.4426950408889634f;
   p.kv_tiles = (const int4*)workspace;
   p.n_kv_tiles = cdiv(a->kv_len, kTileRows);
   hipStream_t stream = (hipStream_t)stream_;
