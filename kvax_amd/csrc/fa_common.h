@@ -7,7 +7,7 @@
 // A C tile can therefore be fed back as a B operand whose contraction index is the C row
 // index: k-slot e of half h in step s (s = 0, 1) is C register 8 * s + e, i.e. row
 // 16 * s + 8 * (e / 4) + 4 * h + e % 4.  The matching A operand gathers those rows with two
-// transposing LDS reads (ds_read_b64_tr_b16), see tr_read_a().
+// transposing LDS reads (ds_read_b64_tr_b16), see tr_read_a_swz().
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -67,42 +67,6 @@ __device__ __forceinline__ typename Tr::vec8 pack8(float a0, float a1, float a2,
 // 4 * (i % 4) + [0, 4)) and lane i receives column i of it.
 __device__ __forceinline__ s16x4 ds_read_tr16(const void* lds_ptr) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(KVAX_LDS(lds_ptr, s16x4));
-}
-
-// A operand (32 x 16) = transpose of a row-major LDS tile X[row][col] (16-bit elements,
-// `stride` bytes per row): A[m][k-slot e] = X[row0 + 8 * (e / 4) + 4 * h + e % 4][col0 + m],
-// the row order that matches a C tile used as B operand (see file header).
-template <class Tr>
-__device__ __forceinline__ typename Tr::vec8 tr_read_a(const char* tile, int stride, int row0,
-                                                       int col0, int lane) {
-  const int g = lane >> 4, i = lane & 15;
-  const int h = g >> 1;
-  const char* p = tile + (row0 + 4 * h + (i >> 2)) * stride + (col0 + 16 * (g & 1) + 4 * (i & 3)) * 2;
-  s16x4 lo = ds_read_tr16(p);
-  s16x4 hi = ds_read_tr16(p + 8 * stride);
-  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  return __builtin_bit_cast(typename Tr::vec8, v);
-}
-
-// Same gather but with the natural k order (k-slot e of half h = row row0 + 8 * h + e): used when
-// the B operand comes from memory rather than from a C tile.
-template <class Tr>
-__device__ __forceinline__ typename Tr::vec8 tr_read_a_linear(const char* tile, int stride,
-                                                              int row0, int col0, int lane) {
-  const int g = lane >> 4, i = lane & 15;
-  const int h = g >> 1;
-  const char* p = tile + (row0 + 8 * h + (i >> 2)) * stride + (col0 + 16 * (g & 1) + 4 * (i & 3)) * 2;
-  s16x4 lo = ds_read_tr16(p);
-  s16x4 hi = ds_read_tr16(p + 4 * stride);
-  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  return __builtin_bit_cast(typename Tr::vec8, v);
-}
-
-// Natural operand read: 8 consecutive elements of row `row` starting at column `col`.
-template <class Tr>
-__device__ __forceinline__ typename Tr::vec8 read_row8(const char* tile, int stride, int row,
-                                                       int col) {
-  return *reinterpret_cast<const typename Tr::vec8*>(tile + row * stride + col * 2);
 }
 
 // v_exp_f32 / v_log_f32 without the denormal-range fix-ups of exp2f / log2f.
@@ -226,29 +190,6 @@ __device__ __forceinline__ void mark_live_tiles(const int4* tiles, const TilePar
     const unsigned long long m = __ballot(live);
     if (lane == 0) bits[w - word0] = m;
   }
-}
-
-// First tile > t_after that is live for any of the NW wavefronts, or INT_MAX.  Uniform.
-template <int NW>
-__device__ __forceinline__ int next_live_tile(const unsigned long long* bits, int words, int word0,
-                                              int t_after) {
-  int t = t_after + 1;
-  int w = max(t >> 6, word0);
-  if (w > (t >> 6)) t = w << 6;
-  while (w - word0 < words) {
-    unsigned long long m = 0;
-#pragma unroll
-    for (int i = 0; i < NW; i++) m |= bits[i * words + (w - word0)];
-    m &= ~0ull << (t & 63);
-    if (m) return (w << 6) + (int)__ffsll((long long)m) - 1;
-    w++;
-    t = w << 6;
-  }
-  return 0x7fffffff;
-}
-
-__device__ __forceinline__ bool tile_is_live(const unsigned long long* wave_bits, int word0, int t) {
-  return (wave_bits[(t >> 6) - word0] >> (t & 63)) & 1;
 }
 
 // Compacts the NW per-wave bitmaps into a list of the tiles that are live for at least one
@@ -424,36 +365,5 @@ __device__ __forceinline__ typename Tr::vec8 tr_read_a_swz(const char* tile_row0
   s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   return __builtin_bit_cast(typename Tr::vec8, v);
 }
-
-// Cooperative staging of a ROWS x D tile of 16-bit elements: global -> registers (issued early
-// so the loads are in flight during compute) -> LDS rows of `lds_stride` bytes.  Rows at or
-// beyond `limit` are zero-filled.
-template <int ROWS, int D, int NT>
-struct RowTile {
-  static constexpr int kChunksPerRow = D / 8;  // 16-byte chunks
-  static constexpr int kPerThread = ROWS * kChunksPerRow / NT;
-  static_assert(ROWS * kChunksPerRow % NT == 0, "tile must split evenly over the work-group");
-  uint4 reg[kPerThread];
-
-  __device__ __forceinline__ void load(const char* base, int64_t row_stride_bytes, int row0,
-                                       int limit, int tid) {
-#pragma unroll
-    for (int i = 0; i < kPerThread; i++) {
-      const int id = tid + i * NT;
-      const int row = row0 + id / kChunksPerRow, ch = id % kChunksPerRow;
-      reg[i] = make_uint4(0, 0, 0, 0);
-      if (row < limit)
-        reg[i] = *reinterpret_cast<const uint4*>(base + (int64_t)row * row_stride_bytes + ch * 16);
-    }
-  }
-  __device__ __forceinline__ void store(char* lds, int lds_stride, int tid) const {
-#pragma unroll
-    for (int i = 0; i < kPerThread; i++) {
-      const int id = tid + i * NT;
-      *reinterpret_cast<uint4*>(lds + (id / kChunksPerRow) * lds_stride + (id % kChunksPerRow) * 16) =
-          reg[i];
-    }
-  }
-};
 
 }  // namespace kvax
