@@ -687,11 +687,15 @@ extern "C" size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* a) {
 extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
                            kvax_stream_t stream_) {
   if (int rc = validate_fa_common(a)) return rc;
-  if (!a->dout || !a->dq || !a->dk || !a->dv) return fail(KVAX_EINVAL, "null gradient pointer");
+  // empty tensors (and the masks over an empty outer axis) may come with null pointers
+  const bool has_q = a->batch > 0 && a->q_len > 0, has_kv = a->batch > 0 && a->kv_len > 0;
+  if ((has_q && (!a->dout || !a->dq)) || (has_kv && (!a->dk || !a->dv)))
+    return fail(KVAX_EINVAL, "null gradient pointer");
   if (a->bwd_query_block <= 0 || a->bwd_kv_block <= 0)
     return fail(KVAX_EINVAL, "backward block sizes must be positive");
   for (int i = 0; i < 4; i++)
-    if (!a->dq_mask[i] || !a->dkdv_mask[i]) return fail(KVAX_EINVAL, "backward masks are missing");
+    if ((has_q && !a->dq_mask[i]) || (has_kv && !a->dkdv_mask[i]))
+      return fail(KVAX_EINVAL, "backward masks are missing");
   const int64_t* strides[] = {a->do_strides, a->dq_strides, a->dk_strides, a->dv_strides};
   for (auto s : strides)
     for (int i = 0; i < 3; i++)

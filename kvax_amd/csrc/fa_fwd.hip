@@ -386,8 +386,10 @@ int validate_fa_common(const kvax_fa_args* a) {
   if (a->dtype != KVAX_BF16 && a->dtype != KVAX_F16)
     return fail(KVAX_EUNSUPPORTED, "dtype %d is not supported (bf16 and f16 are)", a->dtype);
   if (a->flags & ~(KVAX_FA_DKDV_F32 | KVAX_FA_SKIP_DELTA | KVAX_FA_SKIP_DQ | KVAX_FA_SKIP_DKDV)) return fail(KVAX_EINVAL, "unknown bits in flags");
-  if (!a->q || !a->k || !a->v || !a->out || !a->lse || !a->q_pos || !a->q_seg || !a->kv_pos ||
-      !a->kv_seg)
+  // empty tensors may come with null pointers
+  const bool has_q = a->batch > 0 && a->q_len > 0, has_kv = a->batch > 0 && a->kv_len > 0;
+  if ((has_q && (!a->q || !a->out || !a->lse || !a->q_pos || !a->q_seg)) ||
+      (has_kv && (!a->k || !a->v || !a->kv_pos || !a->kv_seg)))
     return fail(KVAX_EINVAL, "null tensor pointer");
   const int64_t* strides[] = {a->q_strides, a->k_strides, a->v_strides, a->o_strides};
   for (auto s : strides)
@@ -417,6 +419,7 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
   if ((uintptr_t)workspace % 16) return fail(KVAX_EINVAL, "workspace must be 16-byte aligned");
   if (a->fwd_query_block <= 0 || a->fwd_kv_block <= 0)
     return fail(KVAX_EINVAL, "forward block sizes must be positive");
+  if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
   for (int i = 0; i < 4; i++)
     if (!a->fwd_mask[i]) return fail(KVAX_EINVAL, "forward mask is missing");
   FwdParams p{};

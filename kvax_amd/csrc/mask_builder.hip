@@ -281,8 +281,6 @@ extern "C" int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const
   int max_outer = 0, max_shards = 1;
   for (int m = 0; m < num_masks; m++) {
     const kvax_mask_desc& d = masks[m];
-    if (!d.lower || !d.upper || !d.lower_full || !d.upper_full)
-      return fail(KVAX_EINVAL, "mask %d: null output pointer", m);
     BoundsJob& j = bp.jobs[m];
     const SummaryKey& qs = keys[qk[m]];
     const SummaryKey& ks = keys[kk[m]];
@@ -293,6 +291,8 @@ extern "C" int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const
     j.inner = (const int4*)workspace + inner.offset;
     j.n_outer = outer.n_blocks;
     j.n_inner_total = inner.n_blocks;
+    if (j.n_outer > 0 && (!d.lower || !d.upper || !d.lower_full || !d.upper_full))
+      return fail(KVAX_EINVAL, "mask %d: null output pointer", m);
     j.num_shards = 1;
     if (num_q_shards > 1) {
       if (q_len % num_q_shards || (q_len / num_q_shards) % d.query_block_size)
