@@ -318,33 +318,43 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
 }
 
 // ---------------------------------------------------------------------------------------------
-// dK/dV: one work-group = NW wavefronts x 32 kv rows of one (batch, kv head); streams the live
-// Q / dO tiles of every query head of the group and accumulates dK^T, dV^T in registers.
+// dK/dV: one work-group = 128 kv rows of one (batch, kv head), 8 wavefronts in 4 pairs.  Both
+// wavefronts of a pair own the same 32 kv rows and share a SIMD; they split the work by role:
+//   P wave:  S = Q K^T, P = exp2(S * c - lse)            -> LDS,   dV^T += dO^T P
+//   S wave:  dP = dO V^T,            (P from LDS) dS = P * (dP - delta),   dK^T += Q^T dS
+// so that each holds one accumulator tile set and one fragment set (K or V) - half the registers
+// of doing both, which is what lets two wavefronts run per SIMD - and so that in both halves of
+// a tile one wavefront of the pair has element-wise work while the other has only MFMAs.
+// The work-group streams the live Q / dO tiles of every query head of the group.
 // ---------------------------------------------------------------------------------------------
 template <int D, int STAGES>
 struct DkdvSmem {
   static constexpr int kTileBytes = kTile * D * 2;  // swizzled, unpadded
   static constexpr int kRowData = 4 * kTile * 4;    // lse, delta, seg, pos
   static constexpr int kStage = 2 * kTileBytes + kRowData;
-  static constexpr int kTotal = STAGES * kStage;
+  static constexpr int kStages = STAGES * kStage;
+  static constexpr int kExchange = 4 * 4096;        // per pair: P of one 64 x 32 tile, 16 bits each
+  static constexpr int kTotal = kStages + kExchange;
 };
 
-template <class Tr, int D, int NW, int WPS, int STAGES>
-__global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdParams p) {
+template <class Tr, int D, int WPS, int STAGES>
+__global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p) {
   using vec8 = typename Tr::vec8;
   using Smem = DkdvSmem<D, STAGES>;
-  constexpr int TKV = NW * 32;
+  constexpr int NW = 8;
+  constexpr int TKV = 128;
   constexpr int KSTEPS = D / 16;
   constexpr int DT = D / 32;
   constexpr int RB = D * 2;
   constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
-  static_assert(STAGES == 4, "two tiles in flight, one being read by the previous unit");
-  static_assert(NW >= 4 && NW % 4 == 0, "one wave per row-data array");
+  static_assert(STAGES == 3, "two tiles in flight, one in use");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
   const int wave = tid / 64, lane = tid % 64;
   const int c = lane % 32, h = lane / 32;
+  const int pair = wave & 3;
+  const bool p_wave = wave < 4;  // role, wave-uniform
 
   // early kv tiles see the most queries under a causal mask: run them first
   int group, kv_tile, member;
@@ -362,8 +372,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
   const int t_hi = r.hi > r.lo ? (r.hi + kTile - 1) / kTile : t_lo;
   const int tf_lo = (r.flo + kTile - 1) / kTile, tf_hi = r.fhi / kTile;
 
-  // per-lane kv column
-  const int kvcol = k0 + wave * 32 + c;
+  // per-lane kv column (the same for both wavefronts of a pair)
+  const int kvcol = k0 + pair * 32 + c;
   const bool in = kvcol < p.kv_len;
   const int kvseg = in ? p.kv_seg[(int64_t)b * p.kv_len + kvcol] : -1;
   const int kvpos = in ? p.kv_pos[(int64_t)b * p.kv_len + kvcol] : 0;
@@ -377,7 +387,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
   TileParts mine[1];
   mine[0] = wave_parts(col_width > 0, kvseg, kvpos);
 
-  // live query tiles of [t_lo, t_hi) (the same for every head of the group)
+  // live query tiles of [t_lo, t_hi) (the same for every head of the group; both wavefronts of a
+  // pair mark the same tiles)
   int* live_count = reinterpret_cast<int*>(smem + Smem::kTotal);
   unsigned long long* live_bits = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal + 16);
   const int word0 = t_lo >> 6;
@@ -392,27 +403,25 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
   const int n_live = *live_count;
   const int steps = n_live * p.group;  // every head of the group walks the same list
 
-  f32x16 dk[DT], dv[DT];
+  f32x16 acc[DT];  // dV^T (P wave) or dK^T (S wave): rows = head dim, columns = the lane's kv row
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) dk[dt][i] = 0.f, dv[dt][i] = 0.f;
+    for (int i = 0; i < 16; i++) acc[dt][i] = 0.f;
 
   if (steps > 0) {
-    vec8 kf[KSTEPS], vf[KSTEPS];
+    // stationary fragments: K (negated when the scale is negative) for the P wave, V for the S wave
+    vec8 frag[KSTEPS];
     {
-      const char* kr = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh + (int64_t)(in ? kvcol : 0) * p.k_ss) * 2;
-      const char* vr = p.v + ((int64_t)b * p.v_sb + (int64_t)kv_head * p.v_sh + (int64_t)(in ? kvcol : 0) * p.v_ss) * 2;
+      const char* base = p_wave ? p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh + (int64_t)(in ? kvcol : 0) * p.k_ss) * 2
+                                : p.v + ((int64_t)b * p.v_sb + (int64_t)kv_head * p.v_sh + (int64_t)(in ? kvcol : 0) * p.v_ss) * 2;
+      const uint32_t sign = p_wave ? p.k_sign : 0u;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ks++) {
-        uint4 u = make_uint4(0, 0, 0, 0), w = make_uint4(0, 0, 0, 0);
-        if (in) {
-          u = *reinterpret_cast<const uint4*>(kr + (16 * ks + 8 * h) * 2);
-          w = *reinterpret_cast<const uint4*>(vr + (16 * ks + 8 * h) * 2);
-        }
-        u.x ^= p.k_sign, u.y ^= p.k_sign, u.z ^= p.k_sign, u.w ^= p.k_sign;
-        kf[ks] = __builtin_bit_cast(vec8, u);
-        vf[ks] = __builtin_bit_cast(vec8, w);
+        uint4 u = make_uint4(0, 0, 0, 0);
+        if (in) u = *reinterpret_cast<const uint4*>(base + (16 * ks + 8 * h) * 2);
+        u.x ^= sign, u.y ^= sign, u.z ^= sign, u.w ^= sign;
+        frag[ks] = __builtin_bit_cast(vec8, u);
       }
     }
     int nat_off[KSTEPS], tr_off[DT][2];
@@ -425,7 +434,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
     }
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
-    const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos
+    const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos (twice over)
     const AsyncTileCopy<kTile, D, NW> copy_q(p.q_ss * 2, wave, lane), copy_do(p.do_ss * 2, wave, lane);
     // step s = (head s / n_live of the group, list entry s % n_live)
     auto issue = [&](int step, uint32_t entry, int stage) {
@@ -444,83 +453,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
     };
     auto entry_of = [&](int step) { return live_list[step % n_live]; };
 
-    // ---- the phases of one unit = 32 query rows (mt) of one tile ------------------------------
-    // A: S = Q K^T and dP = dO V^T (32 MFMAs); operand reads run two contraction steps ahead
-    auto phase_a = [&](const char* qrows, const char* dorows, f32x16& s, f32x16& dp) {
-#pragma unroll
-      for (int i = 0; i < 16; i++) s[i] = 0.f, dp[i] = 0.f;
-      vec8 qa[KSTEPS], da[KSTEPS];
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        qa[ks] = *reinterpret_cast<const vec8*>(qrows + nat_off[ks]);
-        da[ks] = *reinterpret_cast<const vec8*>(dorows + nat_off[ks]);
-      }
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        if (ks + 2 < KSTEPS) {
-          qa[ks + 2] = *reinterpret_cast<const vec8*>(qrows + nat_off[ks + 2]);
-          da[ks + 2] = *reinterpret_cast<const vec8*>(dorows + nat_off[ks + 2]);
-        }
-        s = Tr::mfma(qa[ks], kf[ks], s);
-        dp = Tr::mfma(da[ks], vf[ks], dp);
-      }
-      // issue order: 4 reads ahead, then one read per MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-      for (int i = 0; i < 2 * KSTEPS - 4; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-    };
-    // B + C in one basic block: P = exp2(S * |c| - lse), dS = P * (dP - delta), both rounded to the
-    // input dtype, for the current unit -- together with dV^T += dO^T P, dK^T += Q^T dS of the
-    // previous unit (32 MFMAs fed by transposing reads), so that the exponentials and
-    // conversions issue in the shadow of the MFMAs.
-    auto phase_bc = [&](const float* rows, f32x16& s, f32x16& dp, vec8 (&pb)[2], vec8 (&dsb)[2],
-                        const char* qprev, const char* doprev, const vec8 (&pbp)[2], const vec8 (&dsbp)[2]) {
-      float ls[16], dl[16];
-#pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        const float4 lse4 = *reinterpret_cast<const float4*>(rows + 8 * g4 + 4 * h);
-        const float4 del4 = *reinterpret_cast<const float4*>(rows + kTile + 8 * g4 + 4 * h);
-        ls[4 * g4] = lse4.x, ls[4 * g4 + 1] = lse4.y, ls[4 * g4 + 2] = lse4.z, ls[4 * g4 + 3] = lse4.w;
-        dl[4 * g4] = del4.x, dl[4 * g4 + 1] = del4.y, dl[4 * g4 + 2] = del4.z, dl[4 * g4 + 3] = del4.w;
-      }
-#pragma unroll
-      for (int st = 0; st < 2; st++) {
-#pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
-          const vec8 ad = tr_read_a_swz<Tr>(doprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
-          const vec8 aq = tr_read_a_swz<Tr>(qprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
-          dv[dt] = Tr::mfma(ad, pbp[st], dv[dt]);
-          dk[dt] = Tr::mfma(aq, dsbp[st], dk[dt]);
-          // a quarter of the unit's element-wise work per pair of MFMAs
-          const int i0 = 8 * st + dt * (8 / DT);
-#pragma unroll
-          for (int i = i0; i < i0 + 8 / DT; i++) {
-            s[i] = fast_exp2(__builtin_fmaf(s[i], p.scale_log2_abs, -ls[i]));
-            dp[i] = s[i] * (dp[i] - dl[i]);
-          }
-        }
-        pb[st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
-                           s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
-        dsb[st] = pack8<Tr>(dp[8 * st + 0], dp[8 * st + 1], dp[8 * st + 2], dp[8 * st + 3],
-                            dp[8 * st + 4], dp[8 * st + 5], dp[8 * st + 6], dp[8 * st + 7]);
-      }
-    };
-    // C alone (after the last unit)
-    auto phase_c = [&](const char* qprev, const char* doprev, const vec8 (&pbp)[2], const vec8 (&dsbp)[2]) {
-#pragma unroll
-      for (int st = 0; st < 2; st++)
-#pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
-          const vec8 ad = tr_read_a_swz<Tr>(doprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
-          const vec8 aq = tr_read_a_swz<Tr>(qprev + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
-          dv[dt] = Tr::mfma(ad, pbp[st], dv[dt]);
-          dk[dt] = Tr::mfma(aq, dsbp[st], dk[dt]);
-        }
-    };
+    // P of the pair's current tile, 16-bit floats with a 10-bit mantissa whatever the tensor dtype:
+    // [unit mt][half st] x 64 lanes x 16 bytes, in the lane order of the C tile
+    char* exchange = smem + Smem::kStages + pair * 4096 + lane * 16;
 
     uint32_t e0 = entry_of(0);
     uint32_t e1 = steps > 1 ? entry_of(1) : 0;
@@ -528,21 +463,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
     issue(0, e0, 0);
     if (steps > 1) issue(1, e1, 1);
 
-    // Software pipeline over units: phase C of the previous unit is issued together with phase B
-    // of the current one.  A unit the wave has no part in contributes zero operands; before the
-    // first unit the "previous" operands are zero and point at the first tile, which has landed.
-    vec8 pb_prev[2], dsb_prev[2];
-    const vec8 zero8 = __builtin_bit_cast(vec8, make_uint4(0, 0, 0, 0));
-    pb_prev[0] = pb_prev[1] = dsb_prev[0] = dsb_prev[1] = zero8;
-    const char* q_prev = smem;
-    const char* do_prev = smem + Smem::kTileBytes;
-
     int stage = 0;
     for (int step = 0; step < steps; step++) {
+      // the tile has landed; every wavefront is done with the previous tile and its P
       if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
       const uint32_t e3 = step + 3 < steps ? entry_of(step + 3) : 0;
-      if (step + 2 < steps) issue(step + 2, e2, (stage + 2) % STAGES);
+      if (step + 2 < steps) issue(step + 2, e2, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
       const int t = e0 & 0xffffff;
       const bool active = (e0 >> (24 + wave)) & 1;
       const int qr0 = t * kTile;
@@ -552,62 +479,169 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dkdv_kernel(const BwdPara
       const int32_t* rowids = reinterpret_cast<const int32_t*>(rowdata + 2 * kTile);
       const bool full = t >= tf_lo && t < tf_hi;
 
-      if (!active) {
-        // nothing of this tile concerns the wave: retire the pending unit and carry zero operands
-        phase_c(q_prev, do_prev, pb_prev, dsb_prev);
-        pb_prev[0] = pb_prev[1] = dsb_prev[0] = dsb_prev[1] = zero8;
-        q_prev = qtile;
-        do_prev = dotile;
-      } else {
+      // first half of the tile: 16 MFMAs per wavefront, S = Q K^T (P wave) or dP = dO V^T (S wave),
+      // both 32-row units interleaved; operand reads run four ahead of the MFMAs
+      f32x16 x[2];
+      const char* rows_a = p_wave ? qtile : dotile;
+      if (active) {
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++) {
-          f32x16 s, dp;
-          phase_a(qtile + 32 * mt * RB, dotile + 32 * mt * RB, s, dp);
-          if (!full)  // raw scores: masked -> -inf, so that P = exp2(-inf) = 0 (scale_log2_abs > 0)
-            mask_c_tile<false>(s, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
-                               col_width, -INFINITY);
-          vec8 pb[2], dsb[2];
-          phase_bc(rowdata + 32 * mt, s, dp, pb, dsb, q_prev, do_prev, pb_prev, dsb_prev);
-          pb_prev[0] = pb[0], pb_prev[1] = pb[1], dsb_prev[0] = dsb[0], dsb_prev[1] = dsb[1];
-          q_prev = qtile + 32 * mt * RB;
-          do_prev = dotile + 32 * mt * RB;
+        for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+          for (int i = 0; i < 16; i++) x[mt][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++)
+#pragma unroll
+          for (int mt = 0; mt < 2; mt++)
+            x[mt] = Tr::mfma(*reinterpret_cast<const vec8*>(rows_a + 32 * mt * RB + nat_off[ks]), frag[ks], x[mt]);
+        __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * KSTEPS - 4; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      }
+
+      // operands of the second half's first unit do not depend on the exchange: request them now
+      const char* rows_t = p_wave ? dotile : qtile;
+      vec8 ta[2][DT];
+      if (active) {
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++)
+            ta[st][dt] = tr_read_a_swz<Tr>(rows_t + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
+      }
+
+      if (p_wave) {
+        vec8 pb[2][2];
+        if (active) {
+#pragma unroll
+          for (int mt = 0; mt < 2; mt++) {
+            f32x16& sc = x[mt];
+            if (!full)  // raw scores: masked -> -inf, so that P = exp2(-inf) = 0 (scale_log2_abs > 0)
+              mask_c_tile<false>(sc, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
+                                 col_width, -INFINITY);
+#pragma unroll
+            for (int g4 = 0; g4 < 4; g4++) {
+              const float4 l4 = *reinterpret_cast<const float4*>(rowdata + 32 * mt + 8 * g4 + 4 * h);
+              sc[4 * g4 + 0] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 0], p.scale_log2_abs, -l4.x));
+              sc[4 * g4 + 1] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 1], p.scale_log2_abs, -l4.y));
+              sc[4 * g4 + 2] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 2], p.scale_log2_abs, -l4.z));
+              sc[4 * g4 + 3] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 3], p.scale_log2_abs, -l4.w));
+            }
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+              pb[mt][st] = pack8<Tr>(sc[8 * st + 0], sc[8 * st + 1], sc[8 * st + 2], sc[8 * st + 3],
+                                     sc[8 * st + 4], sc[8 * st + 5], sc[8 * st + 6], sc[8 * st + 7]);
+              const uint4 e = make_uint4(F16::pack2(sc[8 * st + 0], sc[8 * st + 1]), F16::pack2(sc[8 * st + 2], sc[8 * st + 3]),
+                                         F16::pack2(sc[8 * st + 4], sc[8 * st + 5]), F16::pack2(sc[8 * st + 6], sc[8 * st + 7]));
+              *reinterpret_cast<uint4*>(exchange + (2 * mt + st) * 1024) = e;
+            }
+          }
+        }
+        __syncthreads();  // P is visible to the S wave
+        if (active) {
+          // dV^T += dO^T P
+#pragma unroll
+          for (int mt = 0; mt < 2; mt++) {
+            vec8 tb[2][DT];
+            if (mt == 0) {
+#pragma unroll
+              for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+                  tb[st][dt] = tr_read_a_swz<Tr>(rows_t + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+            }
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+#pragma unroll
+              for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], pb[mt][st], acc[dt]);
+            if (mt == 0) {
+#pragma unroll
+              for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) ta[st][dt] = tb[st][dt];
+            }
+          }
+        }
+      } else {
+        __syncthreads();  // P of this tile has been written
+        if (active) {
+#pragma unroll
+          for (int mt = 0; mt < 2; mt++) {
+            // dS = P * (dP - delta), rounded to the input dtype; masked entries have P = 0
+            vec8 dsb[2];
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+              const uint4 e = *reinterpret_cast<const uint4*>(exchange + (2 * mt + st) * 1024);
+              const uint32_t w[4] = {e.x, e.y, e.z, e.w};
+              const float4 d0 = *reinterpret_cast<const float4*>(rowdata + kTile + 32 * mt + 8 * (2 * st) + 4 * h);
+              const float4 d1 = *reinterpret_cast<const float4*>(rowdata + kTile + 32 * mt + 8 * (2 * st + 1) + 4 * h);
+              const float dl[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+              float ds[8];
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                ds[2 * j] = F16::to_float((uint16_t)(w[j] & 0xffff)) * (x[mt][8 * st + 2 * j] - dl[2 * j]);
+                ds[2 * j + 1] = F16::to_float((uint16_t)(w[j] >> 16)) * (x[mt][8 * st + 2 * j + 1] - dl[2 * j + 1]);
+              }
+              dsb[st] = pack8<Tr>(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+            }
+            // operands of the next unit, requested before this unit's MFMAs
+            vec8 tb[2][DT];
+            if (mt == 0) {
+#pragma unroll
+              for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++)
+                  tb[st][dt] = tr_read_a_swz<Tr>(rows_t + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+            }
+            // dK^T += Q^T dS
+#pragma unroll
+            for (int st = 0; st < 2; st++)
+#pragma unroll
+              for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], dsb[st], acc[dt]);
+            if (mt == 0) {
+#pragma unroll
+              for (int st = 0; st < 2; st++)
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) ta[st][dt] = tb[st][dt];
+            }
+          }
         }
       }
       e0 = e1, e1 = e2, e2 = e3;
       stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
-    phase_c(q_prev, do_prev, pb_prev, dsb_prev);
   }
 
-  if (in && p.dkdv_f32) {
-    float* krow = reinterpret_cast<float*>(p.dk) + (int64_t)b * p.dk_sb + (int64_t)kv_head * p.dk_sh + (int64_t)kvcol * p.dk_ss;
-    float* vrow = reinterpret_cast<float*>(p.dv) + (int64_t)b * p.dv_sb + (int64_t)kv_head * p.dv_sh + (int64_t)kvcol * p.dv_ss;
+  // ---- epilogue: the P wave holds dV^T, the S wave dK^T (times the scale) ----------------------
+  if (in) {
+    const float mul = p_wave ? 1.f : p.scale;
+    char* base = p_wave ? p.dv : p.dk;
+    const int64_t sb = p_wave ? p.dv_sb : p.dk_sb, sh = p_wave ? p.dv_sh : p.dk_sh, ss = p_wave ? p.dv_ss : p.dk_ss;
+    const int64_t off = (int64_t)b * sb + (int64_t)kv_head * sh + (int64_t)kvcol * ss;
+    if (p.dkdv_f32) {
+      float* row = reinterpret_cast<float*>(base) + off;
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+      for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        const int d0 = 32 * dt + 8 * g4 + 4 * h;
-        *reinterpret_cast<float4*>(krow + d0) =
-            make_float4(dk[dt][4 * g4 + 0] * p.scale, dk[dt][4 * g4 + 1] * p.scale,
-                        dk[dt][4 * g4 + 2] * p.scale, dk[dt][4 * g4 + 3] * p.scale);
-        *reinterpret_cast<float4*>(vrow + d0) =
-            make_float4(dv[dt][4 * g4 + 0], dv[dt][4 * g4 + 1], dv[dt][4 * g4 + 2], dv[dt][4 * g4 + 3]);
-      }
-  } else if (in) {
-    char* krow = p.dk + ((int64_t)b * p.dk_sb + (int64_t)kv_head * p.dk_sh + (int64_t)kvcol * p.dk_ss) * 2;
-    char* vrow = p.dv + ((int64_t)b * p.dv_sb + (int64_t)kv_head * p.dv_sh + (int64_t)kvcol * p.dv_ss) * 2;
+        for (int g4 = 0; g4 < 4; g4++)
+          *reinterpret_cast<float4*>(row + 32 * dt + 8 * g4 + 4 * h) =
+              make_float4(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul, acc[dt][4 * g4 + 2] * mul,
+                          acc[dt][4 * g4 + 3] * mul);
+    } else {
+      char* row = base + off * 2;
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+      for (int dt = 0; dt < DT; dt++)
 #pragma unroll
-      for (int g4 = 0; g4 < 4; g4++) {
-        uint2 u, w;
-        u.x = Tr::pack2(dk[dt][4 * g4 + 0] * p.scale, dk[dt][4 * g4 + 1] * p.scale);
-        u.y = Tr::pack2(dk[dt][4 * g4 + 2] * p.scale, dk[dt][4 * g4 + 3] * p.scale);
-        w.x = Tr::pack2(dv[dt][4 * g4 + 0], dv[dt][4 * g4 + 1]);
-        w.y = Tr::pack2(dv[dt][4 * g4 + 2], dv[dt][4 * g4 + 3]);
-        *reinterpret_cast<uint2*>(krow + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
-        *reinterpret_cast<uint2*>(vrow + (32 * dt + 8 * g4 + 4 * h) * 2) = w;
-      }
+        for (int g4 = 0; g4 < 4; g4++) {
+          uint2 u;
+          u.x = Tr::pack2(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul);
+          u.y = Tr::pack2(acc[dt][4 * g4 + 2] * mul, acc[dt][4 * g4 + 3] * mul);
+          *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
+        }
+    }
   }
 }
 
@@ -654,14 +688,14 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
   }
-  // dK/dV: 4 wavefronts (128 kv rows) per work-group, one per SIMD
+  // dK/dV: 8 wavefronts in 4 role pairs (128 kv rows) per work-group, two per SIMD
   if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
-    constexpr int NW = 4;
-    auto kernel = fa_bwd_dkdv_kernel<Tr, D, NW, 1, 4>;
+    constexpr int NW = 8;
+    auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2, 3>;
     static bool done = false;
-    const int smem = DkdvSmem<D, 4>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
+    const int smem = DkdvSmem<D, 3>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
     if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
-    p.num_tiles = cdiv(p.kv_len, NW * 32);
+    p.num_tiles = cdiv(p.kv_len, 128);
     p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, 1}.grid();
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dkdv_kernel")) return rc;
