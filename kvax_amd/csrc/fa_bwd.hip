@@ -320,34 +320,39 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
 // ---------------------------------------------------------------------------------------------
 // dK/dV: one work-group = 128 kv rows of one (batch, kv head), 8 wavefronts in 4 pairs.  Both
 // wavefronts of a pair own the same 32 kv rows and share a SIMD; they split the work by role:
-//   P wave:  S = Q K^T, P = exp2(S * c - lse)            -> LDS,   dV^T += dO^T P
-//   S wave:  dP = dO V^T,            (P from LDS) dS = P * (dP - delta),   dK^T += Q^T dS
+//   P wave, tile t:  S = Q K^T,  P = exp2(S * c - lse) -> LDS,  dV^T += dO^T P
+//   S wave, tile t:  dS = P * (dP - delta) and dK^T += Q^T dS of tile t - 1 (P from LDS, dP kept
+//                    in registers), then dP = dO V^T of tile t
 // so that each holds one accumulator tile set and one fragment set (K or V) - half the registers
-// of doing both, which is what lets two wavefronts run per SIMD - and so that in both halves of
-// a tile one wavefront of the pair has element-wise work while the other has only MFMAs.
-// The work-group streams the live Q / dO tiles of every query head of the group.
+// of doing both, which is what lets two wavefronts run per SIMD.  The S wave running one tile
+// behind means one barrier per tile, and at any time one wavefront of the pair has element-wise
+// work while the other has MFMAs.  The work-group streams the live Q / dO tiles of every query
+// head of the group; Q tiles stay one step longer than dO tiles, hence separate rings.
 // ---------------------------------------------------------------------------------------------
-template <int D, int STAGES>
+template <int D>
 struct DkdvSmem {
   static constexpr int kTileBytes = kTile * D * 2;  // swizzled, unpadded
   static constexpr int kRowData = 4 * kTile * 4;    // lse, delta, seg, pos
-  static constexpr int kStage = 2 * kTileBytes + kRowData;
-  static constexpr int kStages = STAGES * kStage;
-  static constexpr int kExchange = 4 * 4096;        // per pair: P of one 64 x 32 tile, 16 bits each
-  static constexpr int kTotal = kStages + kExchange;
+  static constexpr int kQStages = 4, kDoStages = 3;
+  static constexpr int kQ = 0;
+  static constexpr int kDo = kQ + kQStages * kTileBytes;
+  static constexpr int kRows = kDo + kDoStages * kTileBytes;
+  static constexpr int kExchange = kRows + kQStages * kRowData;
+  // per pair two slots of P (one 64 x 32 tile, 16 bits per element): written for tile t while the
+  // slot of tile t - 1 is read
+  static constexpr int kTotal = kExchange + 4 * 2 * 4096;
 };
 
-template <class Tr, int D, int WPS, int STAGES>
+template <class Tr, int D, int WPS>
 __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p) {
   using vec8 = typename Tr::vec8;
-  using Smem = DkdvSmem<D, STAGES>;
+  using Smem = DkdvSmem<D>;
   constexpr int NW = 8;
   constexpr int TKV = 128;
   constexpr int KSTEPS = D / 16;
   constexpr int DT = D / 32;
   constexpr int RB = D * 2;
   constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
-  static_assert(STAGES == 3, "two tiles in flight, one in use");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -436,52 +441,109 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
     const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos (twice over)
     const AsyncTileCopy<kTile, D, NW> copy_q(p.q_ss * 2, wave, lane), copy_do(p.do_ss * 2, wave, lane);
-    // step s = (head s / n_live of the group, list entry s % n_live)
-    auto issue = [&](int step, uint32_t entry, int stage) {
+    // step s = (head s / n_live of the group, list entry s % n_live); its Q tile and row data go to
+    // slot s % 4 of their rings, its dO tile to slot s % 3
+    auto issue = [&](int step, uint32_t entry, int q_slot, int do_slot) {
       const int head = kv_head * p.group + step / n_live;
       const int qr0 = (int)(entry & 0xffffff) * kTile;
-      const uint32_t base = smem_addr + stage * Smem::kStage;
-      copy_q(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, qr0, p.q_len, base);
-      copy_do(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, qr0, p.q_len, base + Smem::kTileBytes);
+      copy_q(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, qr0, p.q_len,
+             smem_addr + Smem::kQ + q_slot * Smem::kTileBytes);
+      copy_do(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, qr0, p.q_len,
+              smem_addr + Smem::kDo + do_slot * Smem::kTileBytes);
       const int qi = min(qr0 + lane, p.q_len - 1);
       const int64_t hoff = ((int64_t)b * p.num_heads + head) * p.q_len + qi;
       const int64_t boff = (int64_t)b * p.q_len + qi;
       const void* src = which == 0 ? (const void*)(p.lse + hoff)
                       : which == 1 ? (const void*)(p.delta + hoff)
                       : which == 2 ? (const void*)(p.q_seg + boff) : (const void*)(p.q_pos + boff);
-      async_copy_b32(src, __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + which * (kTile * 4)));
+      async_copy_b32(src, __builtin_amdgcn_readfirstlane(smem_addr + Smem::kRows + q_slot * Smem::kRowData +
+                                                         which * (kTile * 4)));
     };
     auto entry_of = [&](int step) { return live_list[step % n_live]; };
 
-    // P of the pair's current tile, 16-bit floats with a 10-bit mantissa whatever the tensor dtype:
-    // [unit mt][half st] x 64 lanes x 16 bytes, in the lane order of the C tile
-    char* exchange = smem + Smem::kStages + pair * 4096 + lane * 16;
+    // P of the pair's tiles, 16-bit floats with a 10-bit mantissa whatever the tensor dtype:
+    // [slot][unit mt][half st] x 64 lanes x 16 bytes, in the lane order of the C tile
+    char* exchange = smem + Smem::kExchange + pair * 8192 + lane * 16;
+
+    // S wave, second part of a tile: dS = P * (dP - delta) rounded to the input dtype (masked
+    // entries have P = 0), dK^T += Q^T dS.  x = dP of that tile.
+    auto finish_dk = [&](const f32x16 (&x)[2], const char* qtile, const float* delta_rows, const char* pslot) {
+      vec8 ta[2][DT];
+#pragma unroll
+      for (int st = 0; st < 2; st++)
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+          ta[st][dt] = tr_read_a_swz<Tr>(qtile + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
+#pragma unroll
+      for (int mt = 0; mt < 2; mt++) {
+        vec8 dsb[2];
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+          const uint4 e = *reinterpret_cast<const uint4*>(pslot + (2 * mt + st) * 1024);
+          const uint32_t w[4] = {e.x, e.y, e.z, e.w};
+          const float4 d0 = *reinterpret_cast<const float4*>(delta_rows + 32 * mt + 8 * (2 * st) + 4 * h);
+          const float4 d1 = *reinterpret_cast<const float4*>(delta_rows + 32 * mt + 8 * (2 * st + 1) + 4 * h);
+          const float dl[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+          float ds[8];
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            ds[2 * j] = F16::to_float((uint16_t)(w[j] & 0xffff)) * (x[mt][8 * st + 2 * j] - dl[2 * j]);
+            ds[2 * j + 1] = F16::to_float((uint16_t)(w[j] >> 16)) * (x[mt][8 * st + 2 * j + 1] - dl[2 * j + 1]);
+          }
+          dsb[st] = pack8<Tr>(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+        }
+        vec8 tb[2][DT];  // operands of the next unit, requested before this unit's MFMAs
+        if (mt == 0) {
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+              tb[st][dt] = tr_read_a_swz<Tr>(qtile + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+        }
+#pragma unroll
+        for (int st = 0; st < 2; st++)
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], dsb[st], acc[dt]);
+        if (mt == 0) {
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) ta[st][dt] = tb[st][dt];
+        }
+      }
+    };
 
     uint32_t e0 = entry_of(0);
     uint32_t e1 = steps > 1 ? entry_of(1) : 0;
     uint32_t e2 = steps > 2 ? entry_of(2) : 0;
-    issue(0, e0, 0);
-    if (steps > 1) issue(1, e1, 1);
+    uint32_t ep = 0;  // entry of the previous step
+    issue(0, e0, 0, 0);
+    if (steps > 1) issue(1, e1, 1, 1);
 
-    int stage = 0;
+    f32x16 x[2];  // S of this tile (P wave) / dP carried from the previous step (S wave)
+    int q_slot = 0, do_slot = 0, q_prev = 0;
     for (int step = 0; step < steps; step++) {
-      // the tile has landed; every wavefront is done with the previous tile and its P
+      // the tile has landed; every wavefront is done with the previous step
       if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
       const uint32_t e3 = step + 3 < steps ? entry_of(step + 3) : 0;
-      if (step + 2 < steps) issue(step + 2, e2, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      if (step + 2 < steps) issue(step + 2, e2, (q_slot + 2) & 3, do_slot >= 1 ? do_slot - 1 : 2);
       const int t = e0 & 0xffffff;
-      const bool active = (e0 >> (24 + wave)) & 1;
+      const bool active = (e0 >> (24 + wave)) & 1, active_prev = (ep >> (24 + wave)) & 1;
       const int qr0 = t * kTile;
-      const char* qtile = smem + stage * Smem::kStage;
-      const char* dotile = qtile + Smem::kTileBytes;
-      const float* rowdata = reinterpret_cast<const float*>(qtile + 2 * Smem::kTileBytes);
+      const char* qtile = smem + Smem::kQ + q_slot * Smem::kTileBytes;
+      const char* dotile = smem + Smem::kDo + do_slot * Smem::kTileBytes;
+      const float* rowdata = reinterpret_cast<const float*>(smem + Smem::kRows + q_slot * Smem::kRowData);
       const int32_t* rowids = reinterpret_cast<const int32_t*>(rowdata + 2 * kTile);
       const bool full = t >= tf_lo && t < tf_hi;
 
-      // first half of the tile: 16 MFMAs per wavefront, S = Q K^T (P wave) or dP = dO V^T (S wave),
-      // both 32-row units interleaved; operand reads run four ahead of the MFMAs
-      f32x16 x[2];
+      if (!p_wave && active_prev)
+        finish_dk(x, smem + Smem::kQ + q_prev * Smem::kTileBytes,
+                  reinterpret_cast<const float*>(smem + Smem::kRows + q_prev * Smem::kRowData) + kTile,
+                  exchange + ((step - 1) & 1) * 4096);
+
+      // 16 MFMAs per wavefront, S = Q K^T (P wave) or dP = dO V^T (S wave), both 32-row units
+      // interleaved; operand reads run four ahead of the MFMAs
       const char* rows_a = p_wave ? qtile : dotile;
       if (active) {
 #pragma unroll
@@ -502,117 +564,73 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
         __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
       }
 
-      // operands of the second half's first unit do not depend on the exchange: request them now
-      const char* rows_t = p_wave ? dotile : qtile;
-      vec8 ta[2][DT];
-      if (active) {
+      if (p_wave && active) {
+        // operands of dV's first unit, requested before the element-wise work
+        vec8 ta[2][DT];
 #pragma unroll
         for (int st = 0; st < 2; st++)
 #pragma unroll
           for (int dt = 0; dt < DT; dt++)
-            ta[st][dt] = tr_read_a_swz<Tr>(rows_t + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
-      }
-
-      if (p_wave) {
+            ta[st][dt] = tr_read_a_swz<Tr>(dotile + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
         vec8 pb[2][2];
-        if (active) {
+        char* pslot = exchange + (step & 1) * 4096;
 #pragma unroll
-          for (int mt = 0; mt < 2; mt++) {
-            f32x16& sc = x[mt];
-            if (!full)  // raw scores: masked -> -inf, so that P = exp2(-inf) = 0 (scale_log2_abs > 0)
-              mask_c_tile<false>(sc, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
-                                 col_width, -INFINITY);
+        for (int mt = 0; mt < 2; mt++) {
+          f32x16& sc = x[mt];
+          if (!full)  // raw scores: masked -> -inf, so that P = exp2(-inf) = 0 (scale_log2_abs > 0)
+            mask_c_tile<false>(sc, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
+                               col_width, -INFINITY);
 #pragma unroll
-            for (int g4 = 0; g4 < 4; g4++) {
-              const float4 l4 = *reinterpret_cast<const float4*>(rowdata + 32 * mt + 8 * g4 + 4 * h);
-              sc[4 * g4 + 0] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 0], p.scale_log2_abs, -l4.x));
-              sc[4 * g4 + 1] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 1], p.scale_log2_abs, -l4.y));
-              sc[4 * g4 + 2] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 2], p.scale_log2_abs, -l4.z));
-              sc[4 * g4 + 3] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 3], p.scale_log2_abs, -l4.w));
-            }
+          for (int g4 = 0; g4 < 4; g4++) {
+            const float4 l4 = *reinterpret_cast<const float4*>(rowdata + 32 * mt + 8 * g4 + 4 * h);
+            sc[4 * g4 + 0] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 0], p.scale_log2_abs, -l4.x));
+            sc[4 * g4 + 1] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 1], p.scale_log2_abs, -l4.y));
+            sc[4 * g4 + 2] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 2], p.scale_log2_abs, -l4.z));
+            sc[4 * g4 + 3] = fast_exp2(__builtin_fmaf(sc[4 * g4 + 3], p.scale_log2_abs, -l4.w));
+          }
 #pragma unroll
-            for (int st = 0; st < 2; st++) {
-              pb[mt][st] = pack8<Tr>(sc[8 * st + 0], sc[8 * st + 1], sc[8 * st + 2], sc[8 * st + 3],
-                                     sc[8 * st + 4], sc[8 * st + 5], sc[8 * st + 6], sc[8 * st + 7]);
-              const uint4 e = make_uint4(F16::pack2(sc[8 * st + 0], sc[8 * st + 1]), F16::pack2(sc[8 * st + 2], sc[8 * st + 3]),
-                                         F16::pack2(sc[8 * st + 4], sc[8 * st + 5]), F16::pack2(sc[8 * st + 6], sc[8 * st + 7]));
-              *reinterpret_cast<uint4*>(exchange + (2 * mt + st) * 1024) = e;
-            }
+          for (int st = 0; st < 2; st++) {
+            pb[mt][st] = pack8<Tr>(sc[8 * st + 0], sc[8 * st + 1], sc[8 * st + 2], sc[8 * st + 3],
+                                   sc[8 * st + 4], sc[8 * st + 5], sc[8 * st + 6], sc[8 * st + 7]);
+            const uint4 e = make_uint4(F16::pack2(sc[8 * st + 0], sc[8 * st + 1]), F16::pack2(sc[8 * st + 2], sc[8 * st + 3]),
+                                       F16::pack2(sc[8 * st + 4], sc[8 * st + 5]), F16::pack2(sc[8 * st + 6], sc[8 * st + 7]));
+            *reinterpret_cast<uint4*>(pslot + (2 * mt + st) * 1024) = e;
           }
         }
-        __syncthreads();  // P is visible to the S wave
-        if (active) {
-          // dV^T += dO^T P
+        // dV^T += dO^T P
 #pragma unroll
-          for (int mt = 0; mt < 2; mt++) {
-            vec8 tb[2][DT];
-            if (mt == 0) {
-#pragma unroll
-              for (int st = 0; st < 2; st++)
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++)
-                  tb[st][dt] = tr_read_a_swz<Tr>(rows_t + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
-            }
+        for (int mt = 0; mt < 2; mt++) {
+          vec8 tb[2][DT];
+          if (mt == 0) {
 #pragma unroll
             for (int st = 0; st < 2; st++)
 #pragma unroll
-              for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], pb[mt][st], acc[dt]);
-            if (mt == 0) {
-#pragma unroll
-              for (int st = 0; st < 2; st++)
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++) ta[st][dt] = tb[st][dt];
-            }
+              for (int dt = 0; dt < DT; dt++)
+                tb[st][dt] = tr_read_a_swz<Tr>(dotile + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
           }
-        }
-      } else {
-        __syncthreads();  // P of this tile has been written
-        if (active) {
 #pragma unroll
-          for (int mt = 0; mt < 2; mt++) {
-            // dS = P * (dP - delta), rounded to the input dtype; masked entries have P = 0
-            vec8 dsb[2];
+          for (int st = 0; st < 2; st++)
 #pragma unroll
-            for (int st = 0; st < 2; st++) {
-              const uint4 e = *reinterpret_cast<const uint4*>(exchange + (2 * mt + st) * 1024);
-              const uint32_t w[4] = {e.x, e.y, e.z, e.w};
-              const float4 d0 = *reinterpret_cast<const float4*>(rowdata + kTile + 32 * mt + 8 * (2 * st) + 4 * h);
-              const float4 d1 = *reinterpret_cast<const float4*>(rowdata + kTile + 32 * mt + 8 * (2 * st + 1) + 4 * h);
-              const float dl[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
-              float ds[8];
-#pragma unroll
-              for (int j = 0; j < 4; j++) {
-                ds[2 * j] = F16::to_float((uint16_t)(w[j] & 0xffff)) * (x[mt][8 * st + 2 * j] - dl[2 * j]);
-                ds[2 * j + 1] = F16::to_float((uint16_t)(w[j] >> 16)) * (x[mt][8 * st + 2 * j + 1] - dl[2 * j + 1]);
-              }
-              dsb[st] = pack8<Tr>(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
-            }
-            // operands of the next unit, requested before this unit's MFMAs
-            vec8 tb[2][DT];
-            if (mt == 0) {
-#pragma unroll
-              for (int st = 0; st < 2; st++)
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++)
-                  tb[st][dt] = tr_read_a_swz<Tr>(rows_t + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
-            }
-            // dK^T += Q^T dS
+            for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], pb[mt][st], acc[dt]);
+          if (mt == 0) {
 #pragma unroll
             for (int st = 0; st < 2; st++)
 #pragma unroll
-              for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], dsb[st], acc[dt]);
-            if (mt == 0) {
-#pragma unroll
-              for (int st = 0; st < 2; st++)
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++) ta[st][dt] = tb[st][dt];
-            }
+              for (int dt = 0; dt < DT; dt++) ta[st][dt] = tb[st][dt];
           }
         }
       }
-      e0 = e1, e1 = e2, e2 = e3;
-      stage = stage == STAGES - 1 ? 0 : stage + 1;
+      ep = e0, e0 = e1, e1 = e2, e2 = e3;
+      q_prev = q_slot;
+      q_slot = (q_slot + 1) & 3;
+      do_slot = do_slot == 2 ? 0 : do_slot + 1;
     }
+    // the S wave still owes the last tile
+    __syncthreads();
+    if (!p_wave && ((ep >> (24 + wave)) & 1))
+      finish_dk(x, smem + Smem::kQ + q_prev * Smem::kTileBytes,
+                reinterpret_cast<const float*>(smem + Smem::kRows + q_prev * Smem::kRowData) + kTile,
+                exchange + ((steps - 1) & 1) * 4096);
   }
 
   // ---- epilogue: the P wave holds dV^T, the S wave dK^T (times the scale) ----------------------
@@ -691,9 +709,9 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   // dK/dV: 8 wavefronts in 4 role pairs (128 kv rows) per work-group, two per SIMD
   if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
     constexpr int NW = 8;
-    auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2, 3>;
+    auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2>;
     static bool done = false;
-    const int smem = DkdvSmem<D, 3>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
+    const int smem = DkdvSmem<D>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
     if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, 128);
     p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, 1}.grid();
