@@ -263,9 +263,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
         const int32_t* ids = reinterpret_cast<const int32_t*>(ktile + 2 * Smem::kTileBytes);
         const bool full = t >= tf_lo && t < tf_hi;
 
-        vec8 dsb[2][2];
-#pragma unroll
+#pragma unroll 1
         for (int kt = 0; kt < 2; kt++) {
+          // S^T = K Q^T and dP^T = V dO^T for 32 kv rows: 16 MFMAs, operand reads four ahead
           f32x16 s, dp;
 #pragma unroll
           for (int i2 = 0; i2 < 16; i2++) s[i2] = 0.f, dp[i2] = 0.f;
@@ -276,27 +276,35 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
             s = Tr::mfma(ka, qf[ks], s);
             dp = Tr::mfma(va, dof[ks], dp);
           }
+          __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+          for (int i2 = 0; i2 < 2 * KSTEPS - 4; i2++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+          // K^T operands of this block's dQ update, requested before the element-wise work
+          vec8 ta[2][DT];
+#pragma unroll
+          for (int st = 0; st < 2; st++)
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++)
+              ta[st][dt] = tr_read_a_swz<Tr>(ktile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
 #pragma unroll
           for (int i2 = 0; i2 < 16; i2++) s[i2] = fast_exp2(__builtin_fmaf(s[i2], p.scale_log2, -lse_q));
           if (!full)
             mask_c_tile<true>(s, ids, ids + kTile, 32 * kt, kv0, h, qseg, qpos, col_lo, col_width, 0.f);
 #pragma unroll
           for (int i2 = 0; i2 < 16; i2++) s[i2] *= dp[i2] - delta_q;
+          // dQ^T += K^T dS^T
 #pragma unroll
-          for (int st = 0; st < 2; st++)
-            dsb[kt][st] = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
-                                    s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+          for (int st = 0; st < 2; st++) {
+            const vec8 dsb = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
+                                       s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) dq[dt] = Tr::mfma(ta[st][dt], dsb, dq[dt]);
+          }
         }
-        // dQ^T += K^T dS^T
-#pragma unroll
-        for (int kt = 0; kt < 2; kt++)
-#pragma unroll
-          for (int st = 0; st < 2; st++)
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-              const vec8 a = tr_read_a_swz<Tr>(ktile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
-              dq[dt] = Tr::mfma(a, dsb[kt][st], dq[dt]);
-            }
       }
       e0 = e1, e1 = e2, e2 = e3;
       stage = stage == STAGES - 1 ? 0 : stage + 1;
