@@ -284,12 +284,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
           }
           __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
           // K^T operands of this block's dQ update, requested before the element-wise work
-          vec8 ta[2][DT];
+          vec8 ta[DT];
 #pragma unroll
-          for (int st = 0; st < 2; st++)
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++)
-              ta[st][dt] = tr_read_a_swz<Tr>(ktile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+          for (int dt = 0; dt < DT; dt++)
+            ta[dt] = tr_read_a_swz<Tr>(ktile + 32 * kt * RB, tr_off[dt][0], tr_off[dt][1]);
 #pragma unroll
           for (int i2 = 0; i2 < 16; i2++) s[i2] = fast_exp2(__builtin_fmaf(s[i2], p.scale_log2, -lse_q));
           if (!full)
@@ -301,8 +299,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
           for (int st = 0; st < 2; st++) {
             const vec8 dsb = pack8<Tr>(s[8 * st + 0], s[8 * st + 1], s[8 * st + 2], s[8 * st + 3],
                                        s[8 * st + 4], s[8 * st + 5], s[8 * st + 6], s[8 * st + 7]);
+            vec8 tb[DT];  // second half's operands, requested before the first half's MFMAs
+            if (st == 0) {
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) dq[dt] = Tr::mfma(ta[st][dt], dsb, dq[dt]);
+              for (int dt = 0; dt < DT; dt++)
+                tb[dt] = tr_read_a_swz<Tr>(ktile + (32 * kt + 16) * RB, tr_off[dt][0], tr_off[dt][1]);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) dq[dt] = Tr::mfma(ta[dt], dsb, dq[dt]);
+            if (st == 0) {
+#pragma unroll
+              for (int dt = 0; dt < DT; dt++) ta[dt] = tb[dt];
+            }
           }
         }
       }
@@ -449,25 +457,36 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
     const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos (twice over)
     const AsyncTileCopy<kTile, D, NW> copy_q(p.q_ss * 2, wave, lane), copy_do(p.do_ss * 2, wave, lane);
-    // step s = (head s / n_live of the group, list entry s % n_live); its Q tile and row data go to
-    // slot s % 4 of their rings, its dO tile to slot s % 3
-    auto issue = [&](int step, uint32_t entry, int q_slot, int do_slot) {
-      const int head = kv_head * p.group + step / n_live;
-      const int qr0 = (int)(entry & 0xffffff) * kTile;
-      copy_q(p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2, qr0, p.q_len,
-             smem_addr + Smem::kQ + q_slot * Smem::kTileBytes);
-      copy_do(p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh) * 2, qr0, p.q_len,
-              smem_addr + Smem::kDo + do_slot * Smem::kTileBytes);
-      const int qi = min(qr0 + lane, p.q_len - 1);
-      const int64_t hoff = ((int64_t)b * p.num_heads + head) * p.q_len + qi;
-      const int64_t boff = (int64_t)b * p.q_len + qi;
-      const void* src = which == 0 ? (const void*)(p.lse + hoff)
-                      : which == 1 ? (const void*)(p.delta + hoff)
-                      : which == 2 ? (const void*)(p.q_seg + boff) : (const void*)(p.q_pos + boff);
-      async_copy_b32(src, __builtin_amdgcn_readfirstlane(smem_addr + Smem::kRows + q_slot * Smem::kRowData +
-                                                         which * (kTile * 4)));
+    // Step s = (head s / n_live of the group, list entry s % n_live); its Q tile and row data go to
+    // slot s % 4 of their rings, its dO tile to slot s % 3.  The issuing side keeps its own cursor
+    // (list index, per-head base pointers) and advances it by additions only: divisions and 64-bit
+    // multiplies per copy are serial scalar work of the issuing wave.
+    const int head0 = kv_head * p.group;
+    const char* is_q = p.q + ((int64_t)b * p.q_sb + (int64_t)head0 * p.q_sh) * 2;
+    const char* is_do = p.dout + ((int64_t)b * p.do_sb + (int64_t)head0 * p.do_sh) * 2;
+    // row-data array this wave copies: lse, delta (per head) or seg, pos (per batch row)
+    const char* is_rows = which == 0   ? (const char*)(p.lse + ((int64_t)b * p.num_heads + head0) * p.q_len)
+                          : which == 1 ? (const char*)(p.delta + ((int64_t)b * p.num_heads + head0) * p.q_len)
+                          : which == 2 ? (const char*)(p.q_seg + (int64_t)b * p.q_len)
+                                       : (const char*)(p.q_pos + (int64_t)b * p.q_len);
+    const int64_t rows_per_head = which < 2 ? (int64_t)p.q_len * 4 : 0;
+    int is_li = 0;
+    uint32_t is_entry = live_list[0];
+    auto issue_next = [&](int q_slot, int do_slot) {
+      const int qr0 = (int)(is_entry & 0xffffff) * kTile;
+      copy_q(is_q, qr0, p.q_len, smem_addr + Smem::kQ + q_slot * Smem::kTileBytes);
+      copy_do(is_do, qr0, p.q_len, smem_addr + Smem::kDo + do_slot * Smem::kTileBytes);
+      async_copy_b32(is_rows + (int64_t)min(qr0 + lane, p.q_len - 1) * 4,
+                     __builtin_amdgcn_readfirstlane(smem_addr + Smem::kRows + q_slot * Smem::kRowData +
+                                                    which * (kTile * 4)));
+      if (++is_li == n_live) {
+        is_li = 0;
+        is_q += p.q_sh * 2;
+        is_do += p.do_sh * 2;
+        is_rows += rows_per_head;
+      }
+      is_entry = live_list[is_li];
     };
-    auto entry_of = [&](int step) { return live_list[step % n_live]; };
 
     // P of the pair's tiles, 16-bit floats with a 10-bit mantissa whatever the tensor dtype:
     // [slot][unit mt][half st] x 64 lanes x 16 bytes, in the lane order of the C tile
@@ -521,12 +540,11 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
       }
     };
 
-    uint32_t e0 = entry_of(0);
-    uint32_t e1 = steps > 1 ? entry_of(1) : 0;
-    uint32_t e2 = steps > 2 ? entry_of(2) : 0;
-    uint32_t ep = 0;  // entry of the previous step
-    issue(0, e0, 0, 0);
-    if (steps > 1) issue(1, e1, 1, 1);
+    int li = 0;                    // list index of the current step
+    uint32_t e0 = live_list[0];    // its entry
+    uint32_t ep = 0;               // entry of the previous step
+    issue_next(0, 0);
+    if (steps > 1) issue_next(1, 1);
 
     f32x16 x[2];  // S of this tile (P wave) / dP carried from the previous step (S wave)
     int q_slot = 0, do_slot = 0, q_prev = 0;
@@ -534,8 +552,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
       // the tile has landed; every wavefront is done with the previous step
       if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
-      const uint32_t e3 = step + 3 < steps ? entry_of(step + 3) : 0;
-      if (step + 2 < steps) issue(step + 2, e2, (q_slot + 2) & 3, do_slot >= 1 ? do_slot - 1 : 2);
+      if (step + 2 < steps) issue_next((q_slot + 2) & 3, do_slot >= 1 ? do_slot - 1 : 2);
       const int t = e0 & 0xffffff;
       const bool active = (e0 >> (24 + wave)) & 1, active_prev = (ep >> (24 + wave)) & 1;
       const int qr0 = t * kTile;
@@ -628,7 +645,9 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
           }
         }
       }
-      ep = e0, e0 = e1, e1 = e2, e2 = e3;
+      ep = e0;
+      li = li + 1 == n_live ? 0 : li + 1;
+      e0 = live_list[li];
       q_prev = q_slot;
       q_slot = (q_slot + 1) & 3;
       do_slot = do_slot == 2 ? 0 : do_slot + 1;
@@ -760,6 +779,9 @@ extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t worksp
   for (auto s : strides)
     for (int i = 0; i < 3; i++)
       if (s[i] % 8) return fail(KVAX_EINVAL, "strides must be multiples of 8 elements (16 bytes)");
+  for (auto s : strides)
+    if (s[1] < 0 || s[1] >= (1 << 24))
+      return fail(KVAX_EUNSUPPORTED, "sequence stride of %lld elements is outside [0, 2^24)", (long long)s[1]);
   const void* ptrs[] = {a->dout, a->dq, a->dk, a->dv};
   for (auto ptr : ptrs)
     if ((uintptr_t)ptr % 16) return fail(KVAX_EINVAL, "tensor pointers must be 16-byte aligned");

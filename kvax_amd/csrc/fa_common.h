@@ -296,7 +296,9 @@ __device__ __forceinline__ void async_copy_b128(const char* sbase, uint32_t lane
 // `row_stride_bytes` between rows) into a swizzled LDS tile at LDS address `tile_addr`.  Rows at
 // or beyond `limit` (>= 1) are replaced by row limit - 1: callers mask them out by index.
 // Every wave issues ROWS * D * 2 / 1024 / NW copies; the per-lane part of the source address is
-// computed once (in the constructor) and only a scalar base changes from tile to tile.
+// computed once (in the constructor) and only one scalar base changes from tile to tile: scalar
+// address arithmetic per copy is serial work of the issuing wave and showed up as a fifth of the
+// kernels' time before it was reduced to one multiply per tile.
 template <int ROWS, int D, int NW>
 struct AsyncTileCopy {
   static constexpr int kRowsPerCopy = 1024 / (D * 2);  // 4 (D = 128) or 8 (D = 64)
@@ -304,28 +306,28 @@ struct AsyncTileCopy {
   static constexpr int kPerWave = kCopies / NW;
   static constexpr int kChunks = D / 8;
   static_assert(kCopies % NW == 0, "copies must split evenly over the waves");
-  uint32_t lane_off[kPerWave];  // rin * stride + chunk * 16 for each of the wave's copies
+  uint32_t lane_off[kPerWave];  // (row of the lane within the tile) * stride + chunk * 16, per copy
   int64_t stride;
   int wave_u, rin, pos;
 
+  // The whole tile must span less than 4 GiB (ROWS * row_stride_bytes < 2^32; the entry points
+  // check it), so that one scalar base per tile plus 32-bit lane offsets address every copy.
   __device__ __forceinline__ AsyncTileCopy(int64_t row_stride_bytes, int wave, int lane)
       : stride(row_stride_bytes), wave_u(__builtin_amdgcn_readfirstlane(wave)), rin(lane / kChunks),
         pos(lane % kChunks) {
 #pragma unroll
     for (int j = 0; j < kPerWave; j++) {
       const int r = (j * NW + wave_u) * kRowsPerCopy + rin;
-      lane_off[j] = (uint32_t)(rin * row_stride_bytes) + (uint32_t)((pos ^ swz<D>(r)) * 16);
+      lane_off[j] = (uint32_t)(r * row_stride_bytes) + (uint32_t)((pos ^ swz<D>(r)) * 16);
     }
   }
 
   __device__ __forceinline__ void operator()(const char* gbase, int row0, int limit, uint32_t tile_addr) const {
-    if (row0 + ROWS <= limit) {  // whole tile in range (uniform): scalar base + fixed lane offsets
+    if (row0 + ROWS <= limit) {  // whole tile in range (uniform): one scalar base + fixed lane offsets
+      const char* tile_base = gbase + (int64_t)row0 * stride;
+      const uint32_t lds = tile_addr + wave_u * 1024;
 #pragma unroll
-      for (int j = 0; j < kPerWave; j++) {
-        const int grp = j * NW + wave_u;
-        async_copy_b128(gbase + (int64_t)(row0 + grp * kRowsPerCopy) * stride, lane_off[j],
-                        tile_addr + grp * 1024);
-      }
+      for (int j = 0; j < kPerWave; j++) async_copy_b128(tile_base, lane_off[j], lds + j * NW * 1024);
     } else {  // ragged tail: clamp each lane's row
 #pragma unroll
       for (int j = 0; j < kPerWave; j++) {

@@ -395,6 +395,9 @@ int validate_fa_common(const kvax_fa_args* a) {
   for (auto s : strides)
     for (int i = 0; i < 3; i++)
       if (s[i] % 8) return fail(KVAX_EINVAL, "strides must be multiples of 8 elements (16 bytes)");
+  for (auto s : strides)
+    if (s[1] < 0 || s[1] >= (1 << 24))
+      return fail(KVAX_EUNSUPPORTED, "sequence stride of %lld elements is outside [0, 2^24)", (long long)s[1]);
   const void* ptrs[] = {a->q, a->k, a->v, a->out};
   for (auto ptr : ptrs)
     if ((uintptr_t)ptr % 16) return fail(KVAX_EINVAL, "tensor pointers must be 16-byte aligned");
