@@ -165,9 +165,9 @@ def main():
 
     phases = [("fa_fwd_kernel", fwd)]
     if backward:
-        phases += [("fa_bwd_delta_kernel", lambda: bwd(SQ | SK)),
-                   ("fa_bwd_dq_kernel", lambda: bwd(SD | SK)),
-                   ("fa_bwd_dkdv_kernel", lambda: bwd(SD | SQ))]
+        # the dQ kernel also produces delta = rowsum(O * dO), which the dK/dV kernel reads
+        phases += [("fa_bwd_dq_kernel", lambda: bwd(SK)),
+                   ("fa_bwd_dkdv_kernel", lambda: bwd(SQ))]
 
     def step(events=None):
         for i, (_, fn) in enumerate(phases):
@@ -204,8 +204,7 @@ def main():
     # algorithmic FLOPs per launch of each kernel: 2*D per pair and head for every contraction the
     # kernel exists to produce or must recompute (forward: QK^T, PV; dQ: QK^T, dO V^T, dS K;
     # dK/dV: QK^T, dO V^T, P^T dO, dS^T Q)
-    kernel_flops = {"fa_fwd_kernel": f_fwd, "fa_bwd_delta_kernel": 0.0,
-                    "fa_bwd_dq_kernel": 1.5 * f_fwd, "fa_bwd_dkdv_kernel": 2.0 * f_fwd}
+    kernel_flops = {"fa_fwd_kernel": f_fwd, "fa_bwd_dq_kernel": 1.5 * f_fwd, "fa_bwd_dkdv_kernel": 2.0 * f_fwd}
     dominant = max(kernel_ms, key=kernel_ms.get)
     achieved = kernel_flops[dominant] / (kernel_ms[dominant] * 1e-3) / 1e12
     result = {

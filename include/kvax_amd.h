@@ -87,9 +87,11 @@ int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const int32_t* k
 enum {
   KVAX_FA_DKDV_F32 = 1,  /* backward writes dk / dv as fp32 (the reference kernels' output type,
                             flash_attention_triton.py:1729-1730) instead of the dtype of q */
-  /* Backward phase selection, for profiling one kernel at a time.  The phases are the three
-   * launches of the reference's context-parallel path (:1692, :1740, :1778); skipping a phase
-   * leaves its outputs untouched (a skipped delta phase reuses the workspace contents). */
+  /* Backward phase selection, for profiling one kernel at a time.  The reference's
+   * context-parallel path has three launches (:1692 delta, :1740 dQ, :1778 dK/dV); here the dQ
+   * kernel also produces delta (rowsum(O * dO), kept in the workspace for the dK/dV kernel), so
+   * KVAX_FA_SKIP_DELTA is accepted and changes nothing.  Skipping a phase leaves its outputs
+   * untouched; dK/dV alone reuses the delta a previous call left in the same workspace. */
   KVAX_FA_SKIP_DELTA = 16,
   KVAX_FA_SKIP_DQ = 32,
   KVAX_FA_SKIP_DKDV = 64

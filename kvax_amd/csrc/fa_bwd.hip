@@ -1,5 +1,5 @@
-// Flash-attention backward for gfx950: delta pre-pass, dQ kernel (query-stationary) and dK/dV
-// kernel (kv-stationary, all query heads of a GQA group reduced in registers).
+// Flash-attention backward for gfx950: dQ kernel (query-stationary; also produces delta) and dK/dV
+// kernel (kv-stationary, all query heads of a GQA group reduced in registers), run in that order.
 //
 // Semantics: reference kvax/ops/flash_attention_triton.py:373-410 (delta = rowsum(O * dO)),
 // :526-617 / :620-871 (dQ: P = exp2(S * scale * log2e - lse), dS = P * (dP - delta),
@@ -14,7 +14,8 @@
 //   dQ kernel:    S^T, dP^T [kv x q]  ->  dQ^T [d x q]  += K^T [d x kv]  dS^T [kv x q]
 //   dK/dV kernel: S,   dP   [q x kv]  ->  dV^T [d x kv] += dO^T [d x q]  P  [q x kv]
 //                                         dK^T [d x kv] += Q^T  [d x q]  dS [q x kv]
-// Nothing is exchanged between wavefronts, no atomics are used and the result is deterministic.
+// The dK/dV kernel passes P between the two wavefronts of a pair through LDS (see there); no
+// atomics are used and the result is deterministic.
 #include "common.h"
 #include "fa_common.h"
 
@@ -63,38 +64,6 @@ struct BwdParams {
   float scale_log2_abs;  // |scale| * log2(e) > 0, used with K negated when the scale is negative
   uint32_t k_sign;       // 0x80008000 when the scale is negative
 };
-
-// ---------------------------------------------------------------------------------------------
-// delta[b, h, i] = sum_d O[b, i, h, d] * dO[b, i, h, d]
-// ---------------------------------------------------------------------------------------------
-template <class Tr, int D>
-__global__ __launch_bounds__(256) void fa_bwd_delta_kernel(const BwdParams p) {
-  constexpr int kLanesPerRow = D / 8;
-  constexpr int kRowsPerGroup = 256 / kLanesPerRow;
-  const int64_t row = (int64_t)blockIdx.x * kRowsPerGroup + threadIdx.x / kLanesPerRow;
-  const int part = threadIdx.x % kLanesPerRow;
-  const int64_t total = (int64_t)p.batch * p.q_len * p.num_heads;
-  float acc = 0.f;
-  int b = 0, i = 0, hd = 0;
-  if (row < total) {
-    hd = (int)(row % p.num_heads);
-    i = (int)((row / p.num_heads) % p.q_len);
-    b = (int)(row / ((int64_t)p.num_heads * p.q_len));
-    const uint4 o = *reinterpret_cast<const uint4*>(
-        p.out + (b * p.o_sb + i * p.o_ss + hd * p.o_sh) * 2 + part * 16);
-    const uint4 g = *reinterpret_cast<const uint4*>(
-        p.dout + (b * p.do_sb + i * p.do_ss + hd * p.do_sh) * 2 + part * 16);
-    const uint32_t ow[4] = {o.x, o.y, o.z, o.w}, gw[4] = {g.x, g.y, g.z, g.w};
-#pragma unroll
-    for (int w = 0; w < 4; w++) {
-      acc += Tr::to_float((uint16_t)(ow[w] & 0xffff)) * Tr::to_float((uint16_t)(gw[w] & 0xffff));
-      acc += Tr::to_float((uint16_t)(ow[w] >> 16)) * Tr::to_float((uint16_t)(gw[w] >> 16));
-    }
-  }
-#pragma unroll
-  for (int off = kLanesPerRow / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  if (row < total && part == 0) p.delta[((int64_t)b * p.num_heads + hd) * p.q_len + i] = acc;
-}
 
 // ---------------------------------------------------------------------------------------------
 // Merged range of the streamed axis for a work-group that covers several mask blocks of the
@@ -176,12 +145,38 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   const int qpos = in ? p.q_pos[(int64_t)b * p.q_len + qrow] : 0;
   int col_lo = 0;
   unsigned col_width = 0;
-  float lse_q = 0.f, delta_q = 0.f;
+  float lse_q = 0.f;
   if (in && qseg != -1) {
     col_lo = p.dq_mask[0][mbase + qrow / qbs] * kbs;
     col_width = (unsigned)max(min(p.dq_mask[1][mbase + qrow / qbs] * kbs, p.kv_len) - col_lo, 0);
     lse_q = p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
-    delta_q = p.delta[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
+  }
+  // dO fragments (B operand of dP^T = V dO^T): lane holds 8 consecutive head-dim elements per
+  // step, i.e. half of its row; with the same half of O they give delta = rowsum(O * dO)
+  // (reference attn_bwd_preprocess, flash_attention_triton.py:373-410), which is also written out
+  // for the dK/dV kernel.
+  uint4 draw[KSTEPS];
+  float delta_q = 0.f;
+  {
+    const char* dr = p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh + (int64_t)(in ? qrow : 0) * p.do_ss) * 2;
+    const char* orow = p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh + (int64_t)(in ? qrow : 0) * p.o_ss) * 2;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      uint4 o4 = make_uint4(0, 0, 0, 0);
+      draw[ks] = o4;
+      if (in) {
+        draw[ks] = *reinterpret_cast<const uint4*>(dr + (16 * ks + 8 * h) * 2);
+        o4 = *reinterpret_cast<const uint4*>(orow + (16 * ks + 8 * h) * 2);
+      }
+      const uint32_t ow[4] = {o4.x, o4.y, o4.z, o4.w}, gw[4] = {draw[ks].x, draw[ks].y, draw[ks].z, draw[ks].w};
+#pragma unroll
+      for (int w = 0; w < 4; w++) {
+        delta_q += Tr::to_float((uint16_t)(ow[w] & 0xffff)) * Tr::to_float((uint16_t)(gw[w] & 0xffff));
+        delta_q += Tr::to_float((uint16_t)(ow[w] >> 16)) * Tr::to_float((uint16_t)(gw[w] >> 16));
+      }
+    }
+    delta_q += xor32(delta_q);
+    if (in && h == 0) p.delta[((int64_t)b * p.num_heads + head) * p.q_len + qrow] = delta_q;
   }
   TileParts mine[1];
   mine[0] = wave_parts(col_width > 0, qseg, qpos);
@@ -210,16 +205,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
     vec8 qf[KSTEPS], dof[KSTEPS];
     {
       const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
-      const char* dr = p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh + (int64_t)(in ? qrow : 0) * p.do_ss) * 2;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ks++) {
-        uint4 u = make_uint4(0, 0, 0, 0), w = make_uint4(0, 0, 0, 0);
-        if (in) {
-          u = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
-          w = *reinterpret_cast<const uint4*>(dr + (16 * ks + 8 * h) * 2);
-        }
+        uint4 u = make_uint4(0, 0, 0, 0);
+        if (in) u = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
         qf[ks] = __builtin_bit_cast(vec8, u);
-        dof[ks] = __builtin_bit_cast(vec8, w);
+        dof[ks] = __builtin_bit_cast(vec8, draw[ks]);
       }
     }
     int nat_off[KSTEPS], tr_off[DT][2];
@@ -706,15 +697,6 @@ int reserve_lds(K kernel, int need, int bytes, bool* done, const char* what) {
 template <class Tr, int D>
 int launch_bwd(BwdParams p, hipStream_t stream) {
   constexpr int STAGES = 3;
-  // delta
-  if (!(p.flags & KVAX_FA_SKIP_DELTA)) {
-    const int64_t rows = (int64_t)p.batch * p.q_len * p.num_heads;
-    constexpr int kRowsPerGroup = 256 / (D / 8);
-    if (rows > 0)
-      hipLaunchKernelGGL((fa_bwd_delta_kernel<Tr, D>), dim3((unsigned)((rows + kRowsPerGroup - 1) / kRowsPerGroup)),
-                         dim3(256), 0, stream, p);
-    if (int rc = check_launch("fa_bwd_delta_kernel")) return rc;
-  }
   // tile summaries of both sequences (a few microseconds; needed by dQ and dK/dV)
   {
     TileSummaryJob jobs[2] = {{p.kv_pos, p.kv_seg, (void*)p.kv_tiles, p.kv_len},
