@@ -359,11 +359,12 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
   constexpr int KSTEPS = D / 16;
   constexpr int DT = D / 32;
   constexpr int RB = D * 2;
-  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
+  // only the four P waves issue tile copies: they are the ones with slack before the barrier
+  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, 4>() + 1;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
-  const int wave = tid / 64, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;  // wave-uniform on purpose
   const int c = lane % 32, h = lane / 32;
   const int pair = wave & 3;
   const bool p_wave = wave < 4;  // role, wave-uniform
@@ -446,8 +447,8 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     }
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
-    const int which = wave & 3;  // row-data array this wave copies: lse, delta, seg, pos (twice over)
-    const AsyncTileCopy<kTile, D, NW> copy_q(p.q_ss * 2, wave, lane), copy_do(p.do_ss * 2, wave, lane);
+    const int which = pair;  // row-data array this P wave copies: lse, delta, seg, pos
+    const AsyncTileCopy<kTile, D, 4> copy_q(p.q_ss * 2, pair, lane), copy_do(p.do_ss * 2, pair, lane);
     // Step s = (head s / n_live of the group, list entry s % n_live); its Q tile and row data go to
     // slot s % 4 of their rings, its dO tile to slot s % 3.  The issuing side keeps its own cursor
     // (list index, per-head base pointers) and advances it by additions only: divisions and 64-bit
@@ -534,16 +535,20 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     int li = 0;                    // list index of the current step
     uint32_t e0 = live_list[0];    // its entry
     uint32_t ep = 0;               // entry of the previous step
-    issue_next(0, 0);
-    if (steps > 1) issue_next(1, 1);
+    if (p_wave) {
+      issue_next(0, 0);
+      if (steps > 1) issue_next(1, 1);
+    }
 
     f32x16 x[2];  // S of this tile (P wave) / dP carried from the previous step (S wave)
     int q_slot = 0, do_slot = 0, q_prev = 0;
     for (int step = 0; step < steps; step++) {
       // the tile has landed; every wavefront is done with the previous step
-      if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      if (p_wave) {
+        if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      }
       __syncthreads();
-      if (step + 2 < steps) issue_next((q_slot + 2) & 3, do_slot >= 1 ? do_slot - 1 : 2);
+      if (p_wave && step + 2 < steps) issue_next((q_slot + 2) & 3, do_slot >= 1 ? do_slot - 1 : 2);
       const int t = e0 & 0xffffff;
       const bool active = (e0 >> (24 + wave)) & 1, active_prev = (ep >> (24 + wave)) & 1;
       const int qr0 = t * kTile;
