@@ -113,7 +113,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
-  const int wave = tid / 64, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;  // wave-uniform on purpose
   const int c = lane % 32, h = lane / 32;
 
   int group, rank, g;
