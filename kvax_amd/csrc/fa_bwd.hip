@@ -59,6 +59,7 @@ struct BwdParams {
   const int4* kv_tiles;  // tile summaries [batch, n_kv_tiles, 2]
   const int4* q_tiles;   // tile summaries [batch, n_q_tiles, 2]
   int n_kv_tiles, n_q_tiles;
+  int list_tiles;  // dK/dV kernel: query tiles per chunk of the live-tile bookkeeping
   int flags;
   float scale, scale_log2;
   float scale_log2_abs;  // |scale| * log2(e) > 0, used with K negated when the scale is negative
@@ -400,14 +401,24 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
   TileParts mine[1];
   mine[0] = wave_parts(col_width > 0, kvseg, kvpos);
 
-  // live query tiles of [t_lo, t_hi) (the same for every head of the group; both wavefronts of a
-  // pair mark the same tiles)
+  f32x16 acc[DT];  // dV^T (P wave) or dK^T (S wave): rows = head dim, columns = the lane's kv row
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[dt][i] = 0.f;
+
+  // The query range is walked in chunks of at most p.list_tiles tiles, the number whose live-tile
+  // bookkeeping fits in the LDS left over (one chunk unless the query sequence is very long).
   int* live_count = reinterpret_cast<int*>(smem + Smem::kTotal);
   unsigned long long* live_bits = reinterpret_cast<unsigned long long*>(smem + Smem::kTotal + 16);
-  const int word0 = t_lo >> 6;
-  const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
-  const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.n_q_tiles, 64) + 1));
-  mark_live_tiles<false, 1>(p.q_tiles + 2 * (int64_t)b * p.n_q_tiles, mine, t_lo, t_hi,
+  const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.list_tiles, 64) + 1));
+  for (int c_lo = t_lo; c_lo < t_hi; c_lo += p.list_tiles) {
+  const int c_hi = min(c_lo + p.list_tiles, t_hi);
+  // live query tiles of [c_lo, c_hi) (the same for every head of the group; both wavefronts of a
+  // pair mark the same tiles)
+  const int word0 = c_lo >> 6;
+  const int words = ((c_hi - 1) >> 6) - word0 + 1;
+  mark_live_tiles<false, 1>(p.q_tiles + 2 * (int64_t)b * p.n_q_tiles, mine, c_lo, c_hi,
                             live_bits + wave * words, word0, lane);
   __syncthreads();
   if (wave == 0)
@@ -415,12 +426,6 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
   __syncthreads();
   const int n_live = *live_count;
   const int steps = n_live * p.group;  // every head of the group walks the same list
-
-  f32x16 acc[DT];  // dV^T (P wave) or dK^T (S wave): rows = head dim, columns = the lane's kv row
-#pragma unroll
-  for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-    for (int i = 0; i < 16; i++) acc[dt][i] = 0.f;
 
   if (steps > 0) {
     // stationary fragments: K (negated when the scale is negative) for the P wave, V for the S wave
@@ -655,6 +660,8 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
                 reinterpret_cast<const float*>(smem + Smem::kRows + q_prev * Smem::kRowData) + kTile,
                 exchange + ((steps - 1) & 1) * 4096);
   }
+  __syncthreads();  // the next chunk reuses the bookkeeping, the rings and the exchange slots
+  }
 
   // ---- epilogue: the P wave holds dV^T, the S wave dK^T (times the scale) ----------------------
   if (in) {
@@ -725,8 +732,13 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     constexpr int NW = 8;
     auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2>;
     static bool done = false;
-    const int smem = DkdvSmem<D>::kTotal + live_tiles_bytes(NW, p.n_q_tiles);
-    if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dK/dV kernel")) return rc;
+    // live-tile bookkeeping for as many query tiles as the remaining LDS holds (a multiple of 64)
+    constexpr int kLdsLimit = 160 * 1024;
+    int chunk = 64;
+    while (chunk < p.n_q_tiles && DkdvSmem<D>::kTotal + live_tiles_bytes(NW, chunk * 2) <= kLdsLimit) chunk *= 2;
+    p.list_tiles = min(chunk, max(p.n_q_tiles, 1));
+    const int smem = DkdvSmem<D>::kTotal + live_tiles_bytes(NW, p.list_tiles);
+    if (int rc = reserve_lds(kernel, smem, kLdsLimit, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, 128);
     p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, 1}.grid();
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);

@@ -128,3 +128,33 @@ def test_batch_zero(device):
     ids = [torch.zeros(0, 64, dtype=torch.int32, device=device) for _ in range(4)]
     out, dq, dk, dv = _run((q, k, k.clone(), *ids), 0.125)
     assert out.numel() == 0 and dq.numel() == 0 and dk.numel() == 0 and dv.numel() == 0
+
+
+def test_query_sequence_longer_than_one_bookkeeping_chunk(device):
+    """135168 query rows are 2112 tiles of 64: the dK/dV kernel's live-tile bookkeeping takes 2048 tiles
+    per pass, so this runs its chunked path; dK/dV (fp32) against the dense oracle."""
+    from oracle import attention_oracle as ao
+    sq, sk, d = 135168, 256, 128
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn(1, sq, 1, d, generator=g).to(torch.bfloat16).to(device)
+    k = torch.randn(1, sk, 1, d, generator=g).to(torch.bfloat16).to(device)
+    v = torch.randn(1, sk, 1, d, generator=g).to(torch.bfloat16).to(device)
+    dout = (torch.randn(1, sq, 1, d, generator=g) * 0.05).to(torch.bfloat16).to(device)
+    # two documents; queries of each see the keys of their own half; constant positions = bidirectional
+    q_seg = (torch.arange(sq) >= sq // 3).to(torch.int32)[None].to(device)
+    kv_seg = (torch.arange(sk) >= sk // 2).to(torch.int32)[None].to(device)
+    q_pos, kv_pos = torch.zeros_like(q_seg), torch.zeros_like(kv_seg)
+    p = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg, fwd_params=p, bwd_params=p, calc_bwd_mask=True)
+    scale = d ** -0.5
+    out, lse = flash_attention_forward(q, k, v, q_pos, q_seg, kv_pos, kv_seg, masks[0], scale, p, p)
+    dq, dk, dv = flash_attention_backward(q, k, v, q_pos, q_seg, kv_pos, kv_seg, masks[1], masks[2], out, lse,
+                                          dout, scale, p, p, dkdv_fp32=True)
+    f = lambda t: t.float().cpu().numpy()
+    args = (f(q), f(k), f(v), q_pos.cpu().numpy(), q_seg.cpu().numpy(), kv_pos.cpu().numpy(), kv_seg.cpu().numpy(), scale)
+    ref_dq, ref_dk, ref_dv = ao.attention_backward(*args, f(dout), dtype=np.float32, row_block=8192)
+    for name, got, ref in (("dk", dk, ref_dk), ("dv", dv, ref_dv)):
+        err = np.abs(f(got) - ref).max()
+        assert err <= 2e-2 * max(1.0, np.abs(ref).max()), f"{name}: {err} (|ref| max {np.abs(ref).max()})"
+    assert np.abs(f(dq) - ref_dq).max() <= 2e-2
