@@ -8,6 +8,7 @@ int32 ``[batch, shards, n_outer_blocks]``).  The device work is one call into th
 from __future__ import annotations
 
 import ctypes as C
+import logging
 
 import torch
 
@@ -19,6 +20,8 @@ from kvax_amd.utils.common import (
 from kvax_amd.utils.sharding import context_parallel_degree
 from kvax_amd.utils.specs import get_attention_specs
 from kvax_amd.utils.typing import AttentionMask, DeviceArray
+
+logger = logging.getLogger(__name__)
 
 
 def _as_ids(x: DeviceArray, name: str) -> torch.Tensor:
@@ -141,3 +144,64 @@ def calculate_mask_sparsity(
     visited = (mask.upper_bounds.long() - mask.lower_bounds.long()).sum().item()
     batch = mask.lower_bounds.shape[0]
     return visited / (query_seq_len // query_block_size) / (kv_seq_len // kv_block_size) / batch
+
+
+def mask_block_levels(mask: AttentionMask, num_inner_blocks: int, batch_index: int = 0) -> torch.Tensor:
+    """``[n_outer_blocks, num_inner_blocks]`` int8 grid of one batch entry: 0 = block skipped,
+    1 = visited with the element mask, 2 = visited without it.  Shard ``s`` of a context-parallel
+    mask covers the inner blocks ``[s * num_inner_blocks / shards, (s + 1) * num_inner_blocks / shards)``
+    (kvax/ops/mask_creator.py:507-533)."""
+    lower = mask.lower_bounds[batch_index].cpu().long()
+    shards, _ = lower.shape
+    if num_inner_blocks % shards:
+        raise ValueError(f"{num_inner_blocks} inner blocks do not split over {shards} shards")
+    col = torch.arange(num_inner_blocks // shards).view(1, 1, -1)
+
+    def inside(lo, hi):
+        lo = lo[batch_index].cpu().long().unsqueeze(-1)
+        hi = hi[batch_index].cpu().long().unsqueeze(-1)
+        return (col >= lo) & (col < hi)
+
+    visited = inside(mask.lower_bounds, mask.upper_bounds)
+    full = inside(mask.lower_full_bounds, mask.upper_full_bounds) & visited
+    levels = visited.to(torch.int8) + full.to(torch.int8)  # [shards, n_outer, inner/shards]
+    return levels.permute(1, 0, 2).reshape(lower.shape[1], num_inner_blocks)
+
+
+def render_mask(
+    mask: AttentionMask, num_inner_blocks: int, print_only_first_in_batch: bool = True,
+    fit_in_screen: bool = True, max_rows: int = 32, max_columns: int = 64,
+) -> str:
+    """Text picture of a block mask: two characters per cell, solid where every block of the
+    cell is visited without the element mask, blank where every block is skipped, shaded
+    otherwise.  With ``fit_in_screen`` the grid is pooled down to ``max_rows`` x ``max_columns``
+    cells (same picture as kvax/ops/mask_creator.py:493-598 draws)."""
+    batch = mask.lower_bounds.shape[0]
+    text = "Attention masks:\n"
+    for b in range(1 if print_only_first_in_batch else batch):
+        levels = mask_block_levels(mask, num_inner_blocks, b)
+        rows, cols = levels.shape
+        row_step = max(-(-rows // max_rows), 1) if fit_in_screen else 1
+        col_step = max(-(-cols // max_columns), 1) if fit_in_screen else 1
+        # Pool with padding that counts as "skipped", so ragged edge cells read as partial.
+        padded = torch.zeros((-(-rows // row_step) * row_step, -(-cols // col_step) * col_step),
+                             dtype=torch.int8)
+        padded[:rows, :cols] = levels
+        cells = padded.view(padded.shape[0] // row_step, row_step, padded.shape[1] // col_step, col_step)
+        all_full = (cells == 2).all(dim=3).all(dim=1)
+        all_skipped = (cells == 0).all(dim=3).all(dim=1)
+        width = all_full.shape[1]
+        text += "\n  " + "==" * width + "  \n"
+        for full_row, skipped_row in zip(all_full.tolist(), all_skipped.tolist()):
+            line = "".join("██" if f else "  " if s else "░░" for f, s in zip(full_row, skipped_row))
+            text += "||" + line + "||\n"
+        text += "  " + "==" * width + "  \n\n"
+    return text
+
+
+def print_mask(
+    mask: AttentionMask, num_inner_blocks: int, print_only_first_in_batch: bool = True,
+    fit_in_screen: bool = True,
+) -> None:
+    """Log the picture of ``render_mask`` at INFO level (kvax/ops/mask_creator.py:493-598)."""
+    logger.info(render_mask(mask, num_inner_blocks, print_only_first_in_batch, fit_in_screen))

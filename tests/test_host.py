@@ -133,3 +133,47 @@ def test_pad_to_block_size_and_flops_model():
     t = get_multi_head_attention_tflops(2, 1024, 1024, 8, 128, 128, causal=True,
                                         forward_pass=True, backward_pass=True)
     assert t == pytest.approx(2 * 8 * 4 * 128 * 1024 * 1024 * 0.5 * 3.5 / 1e12)
+
+
+def _toy_mask():
+    from kvax_amd.utils.typing import AttentionMask
+
+    # 4 query blocks x 4 kv blocks, causal with two documents of two blocks each.
+    lower = torch.tensor([[[0, 0, 2, 2]]], dtype=torch.int32)
+    upper = torch.tensor([[[1, 2, 3, 4]]], dtype=torch.int32)
+    lower_full = torch.tensor([[[0, 0, 2, 2]]], dtype=torch.int32)
+    upper_full = torch.tensor([[[0, 1, 2, 3]]], dtype=torch.int32)
+    return AttentionMask(lower, upper, lower_full, upper_full)
+
+
+def test_mask_pictures_and_sparsity():
+    from kvax_amd.ops.mask_creator import (
+        calculate_mask_sparsity, mask_block_levels, print_mask, render_mask,
+    )
+
+    mask = _toy_mask()
+    levels = mask_block_levels(mask, 4)
+    assert levels.tolist() == [[1, 0, 0, 0], [2, 1, 0, 0], [0, 0, 1, 0], [0, 0, 2, 1]]
+    text = render_mask(mask, 4)
+    rows = [line[2:-2] for line in text.splitlines() if line.startswith("||")]
+    assert rows == ["░░      ", "██░░    ", "    ░░  ", "    ██░░"]
+    # Pooled 2x2: no cell is uniformly full, the off-diagonal cells are uniformly skipped.
+    pooled = render_mask(mask, 4, max_rows=2, max_columns=2)
+    assert [l[2:-2] for l in pooled.splitlines() if l.startswith("||")] == ["░░  ", "  ░░"]
+    # Blocks in [lower, upper) over all blocks: 6 of 16.
+    assert calculate_mask_sparsity(mask, 64, 64, 256, 256) == pytest.approx(6 / 16)
+    print_mask(mask, 4)  # logs; must not raise
+
+
+def test_mask_picture_of_a_sharded_mask():
+    from kvax_amd.ops.mask_creator import mask_block_levels
+    from kvax_amd.utils.typing import AttentionMask
+
+    # dK/dV-style mask with 2 query shards: bounds are local to each shard's 2 inner blocks.
+    lower = torch.tensor([[[0, 1], [0, 0]]], dtype=torch.int32)
+    upper = torch.tensor([[[2, 2], [1, 2]]], dtype=torch.int32)
+    zeros = torch.zeros_like(lower)
+    levels = mask_block_levels(AttentionMask(lower, upper, zeros, zeros), 4)
+    assert levels.tolist() == [[1, 1, 1, 0], [0, 1, 1, 1]]
+    with pytest.raises(ValueError):
+        mask_block_levels(AttentionMask(lower, upper, zeros, zeros), 3)

@@ -93,3 +93,24 @@ def test_specs_must_be_set(device):
     w = workload("cpu_plumbing")
     with pytest.raises(ValueError):
         create_attention_mask(*_dev(device, w.q_pos, w.q_seg, w.kv_pos, w.kv_seg))
+
+
+def test_mask_diagnostics_on_device_masks(device):
+    from kvax_amd.ops.mask_creator import calculate_mask_sparsity, mask_block_levels, render_mask
+
+    w = workload("dense_causal")
+    params = FlashAttentionParamsConfig(query_block_size=128, kv_block_size=128)
+    with attention_specs(*TP_SPECS):
+        fwd, dq, dkdv = create_attention_mask(*_dev(device, w.q_pos, w.q_seg, w.kv_pos, w.kv_seg),
+                                              fwd_params=params, bwd_params=params,
+                                              calc_bwd_mask=True)
+    n = w.q_len // 128
+    levels = mask_block_levels(fwd, n)
+    want = torch.tril(torch.full((n, n), 2, dtype=torch.int8), -1) + torch.eye(n, dtype=torch.int8)
+    assert torch.equal(levels, want)
+    # The dK/dV mask is the transposed picture: kv block j is visited by query blocks >= j.
+    assert torch.equal(mask_block_levels(dkdv, n), want.T)
+    assert calculate_mask_sparsity(fwd, 128, 128, w.q_len, w.kv_len) == pytest.approx(
+        (n + 1) / (2 * n))
+    lines = [l for l in render_mask(fwd, n).splitlines() if l.startswith("||")]
+    assert len(lines) == min(n, 32) and lines[0].count("█") == 0 and "░" in lines[0]
