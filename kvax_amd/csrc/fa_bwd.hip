@@ -110,7 +110,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   constexpr int DT = D / 32;
   constexpr int RB = D * 2;
   constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, NW>() + 1;
-  static_assert(STAGES == 3, "the loop below keeps two tiles in flight");
+  static_assert(STAGES == 2 || STAGES == 3, "the loop below keeps STAGES - 1 tiles in flight");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -238,14 +238,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
     uint32_t e1 = n_live > 1 ? live_list[1] : 0;
     uint32_t e2 = n_live > 2 ? live_list[2] : 0;
     issue(e0 & 0xffffff, 0);
-    if (n_live > 1) issue(e1 & 0xffffff, 1);
+    if (STAGES == 3 && n_live > 1) issue(e1 & 0xffffff, 1);
 
     int stage = 0;
     for (int i = 0; i < n_live; i++) {
-      if (i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      if (STAGES == 3 && i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
       const uint32_t e3 = i + 3 < n_live ? live_list[i + 3] : 0;
-      if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      if (STAGES == 3) {
+        if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      } else {
+        if (i + 1 < n_live) issue(e1 & 0xffffff, stage ^ 1);
+      }
       const int t = e0 & 0xffffff;
 
       if ((e0 >> (24 + wave)) & 1) {
@@ -706,26 +710,39 @@ int reserve_lds(K kernel, int need, int bytes, bool* done, const char* what) {
   return KVAX_OK;
 }
 
+// dQ launch: NW wavefronts (32 query rows each) per work-group, two per SIMD.
+template <class Tr, int D, int NW, int STAGES>
+int launch_dq(BwdParams p, hipStream_t stream) {
+  auto kernel = fa_bwd_dq_kernel<Tr, D, NW, 2, STAGES>;
+  static bool done = false;
+  constexpr int kLimit = 160 * 1024 / (8 / NW);
+  const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
+  if (int rc = reserve_lds(kernel, smem, kLimit, &done, "the dQ kernel")) return rc;
+  p.num_tiles = cdiv(p.q_len, NW * 32);
+  p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, p.group}.grid();
+  hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
+  return check_launch("fa_bwd_dq_kernel");
+}
+
 template <class Tr, int D>
 int launch_bwd(BwdParams p, hipStream_t stream) {
-  constexpr int STAGES = 3;
   // tile summaries of both sequences (a few microseconds; needed by dQ and dK/dV)
   {
     TileSummaryJob jobs[2] = {{p.kv_pos, p.kv_seg, (void*)p.kv_tiles, p.kv_len},
                               {p.q_pos, p.q_seg, (void*)p.q_tiles, p.q_len}};
     if (int rc = launch_tile_summaries(jobs, 2, p.batch, stream)) return rc;
   }
-  // dQ: 8 wavefronts (256 query rows) per work-group, two per SIMD, one work-group per CU
+  // dQ: two work-groups of four wavefronts per compute unit (each hides the other's prologue,
+  // barriers and final stores) when the tile bitmaps fit beside the smaller ring, else one of eight
   if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
-    constexpr int NW = 8;
-    auto kernel = fa_bwd_dq_kernel<Tr, D, NW, 2, STAGES>;
-    static bool done = false;
-    const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
-    if (int rc = reserve_lds(kernel, smem, 160 * 1024, &done, "the dQ kernel")) return rc;
-    p.num_tiles = cdiv(p.q_len, NW * 32);
-    p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, p.group}.grid();
-    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
-    if (int rc = check_launch("fa_bwd_dq_kernel")) return rc;
+    static const int cfg = getenv("KVAX_DQ_CFG") ? atoi(getenv("KVAX_DQ_CFG")) : 1;
+    constexpr int kStagesSmall = D == 128 ? 2 : 3;
+    const int small = DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
+    if (cfg == 1 && small <= 80 * 1024) {
+      if (int rc = launch_dq<Tr, D, 4, kStagesSmall>(p, stream)) return rc;
+    } else {
+      if (int rc = launch_dq<Tr, D, 8, 3>(p, stream)) return rc;
+    }
   }
   // dK/dV: 8 wavefronts in 4 role pairs (128 kv rows) per work-group, two per SIMD
   if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {

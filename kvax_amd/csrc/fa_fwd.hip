@@ -71,7 +71,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   constexpr int DT = D / 32;      // 32-row tiles of O^T
   constexpr int RB = D * 2;       // bytes per tile row
   constexpr int kCopies = 2 * async_tile_copies_per_wave<kTK, D, NW>() + 1;  // per wave and tile
-  static_assert(STAGES == 3, "the loop below keeps two tiles in flight");
+  static_assert(STAGES == 2 || STAGES == 3, "the loop below keeps STAGES - 1 tiles in flight");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -213,15 +213,19 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     uint32_t e1 = n_live > 1 ? live_list[1] : 0;
     uint32_t e2 = n_live > 2 ? live_list[2] : 0;
     issue(e0 & 0xffffff, 0);
-    if (n_live > 1) issue(e1 & 0xffffff, 1);
+    if (STAGES == 3 && n_live > 1) issue(e1 & 0xffffff, 1);
 
     int stage = 0;
     for (int i = 0; i < n_live; i++) {
       // tile i has landed once at most the copies of tile i + 1 are outstanding
-      if (i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      if (STAGES == 3 && i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
       const uint32_t e3 = i + 3 < n_live ? live_list[i + 3] : 0;
-      if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      if (STAGES == 3) {
+        if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+      } else {
+        if (i + 1 < n_live) issue(e1 & 0xffffff, stage ^ 1);
+      }
       const int t = e0 & 0xffffff;
 
       if ((e0 >> (24 + wave)) & 1) {
@@ -346,9 +350,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   }
 }
 
-template <class Tr, int D, int MQ, int NW, int WPS>
+template <class Tr, int D, int MQ, int NW, int WPS, int STAGES = 3>
 int launch_fwd(const FwdParams& p0, hipStream_t stream) {
-  constexpr int STAGES = 3;
   FwdParams p = p0;
   constexpr int TQ = NW * 32 * MQ;
   p.num_q_tiles = cdiv(p.q_len, TQ);
@@ -370,6 +373,17 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   }
   hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
   return check_launch("fa_fwd_kernel");
+}
+
+// Two work-groups of four wavefronts per compute unit (each hides the other's prologue, barriers
+// and final stores) whenever the tile bitmaps of the sequence fit beside the smaller ring;
+// otherwise one work-group of eight wavefronts.
+template <class Tr, int D>
+int launch_fwd_auto(const FwdParams& p, hipStream_t stream, int cfg) {
+  constexpr int kStagesSmall = D == 128 ? 2 : 3;
+  const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
+  if (cfg == 1 && small <= 80 * 1024) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
+  return launch_fwd<Tr, D, 1, 8, 2, 3>(p, stream);
 }
 
 }  // namespace
@@ -459,7 +473,8 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
   const bool bf16 = a->dtype == KVAX_BF16;
+  static const int cfg = getenv("KVAX_FWD_CFG") ? atoi(getenv("KVAX_FWD_CFG")) : 1;
   if (a->head_dim == 128)
-    return bf16 ? launch_fwd<Bf16, 128, 1, 8, 2>(p, stream) : launch_fwd<F16, 128, 1, 8, 2>(p, stream);
-  return bf16 ? launch_fwd<Bf16, 64, 1, 8, 2>(p, stream) : launch_fwd<F16, 64, 1, 8, 2>(p, stream);
+    return bf16 ? launch_fwd_auto<Bf16, 128>(p, stream, cfg) : launch_fwd_auto<F16, 128>(p, stream, cfg);
+  return bf16 ? launch_fwd_auto<Bf16, 64>(p, stream, cfg) : launch_fwd_auto<F16, 64>(p, stream, cfg);
 }

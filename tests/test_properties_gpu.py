@@ -158,3 +158,39 @@ def test_query_sequence_longer_than_one_bookkeeping_chunk(device):
         err = np.abs(f(got) - ref).max()
         assert err <= 2e-2 * max(1.0, np.abs(ref).max()), f"{name}: {err} (|ref| max {np.abs(ref).max()})"
     assert np.abs(f(dq) - ref_dq).max() <= 2e-2
+
+
+def test_key_sequence_too_long_for_two_work_groups_per_cu(device):
+    """With 262144 keys the tile bitmaps no longer fit beside the LDS ring of the configuration that
+    runs two work-groups per compute unit, so forward and dQ take the one-work-group configuration:
+    a chunk of 256 late queries over the whole key sequence against the dense oracle."""
+    from oracle import attention_oracle as ao
+    sq, sk, d = 256, 262144, 128
+    g = torch.Generator().manual_seed(23)
+    q = torch.randn(1, sq, 2, d, generator=g).to(torch.bfloat16).to(device)
+    k = torch.randn(1, sk, 1, d, generator=g).to(torch.bfloat16).to(device)
+    v = torch.randn(1, sk, 1, d, generator=g).to(torch.bfloat16).to(device)
+    dout = torch.randn(1, sq, 2, d, generator=g).to(torch.bfloat16).to(device)
+    kv_pos = torch.arange(sk, dtype=torch.int32)[None].to(device)
+    q_pos = (torch.arange(sq, dtype=torch.int32) + (sk - sq - 1000))[None].to(device)
+    # keys: padding at the front, then two documents; the queries belong to the second one
+    kv_seg = torch.ones(1, sk, dtype=torch.int32)
+    kv_seg[:, :5000] = -1
+    kv_seg[:, 5000:70000] = 0
+    kv_seg = kv_seg.to(device)
+    q_seg = torch.ones(1, sq, dtype=torch.int32, device=device)
+    p = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg, fwd_params=p, bwd_params=p, calc_bwd_mask=True)
+    scale = d ** -0.5
+    out, lse = flash_attention_forward(q, k, v, q_pos, q_seg, kv_pos, kv_seg, masks[0], scale, p, p)
+    dq, dk, dv = flash_attention_backward(q, k, v, q_pos, q_seg, kv_pos, kv_seg, masks[1], masks[2], out, lse,
+                                          dout, scale, p, p, dkdv_fp32=True)
+    f = lambda t: t.float().cpu().numpy()
+    args = (f(q), f(k), f(v), q_pos.cpu().numpy(), q_seg.cpu().numpy(), kv_pos.cpu().numpy(), kv_seg.cpu().numpy(), scale)
+    ref_out = ao.attention_forward(*args, dtype=np.float32)[0]
+    ref_dq, ref_dk, ref_dv = ao.attention_backward(*args, f(dout), dtype=np.float32)
+    assert np.abs(f(out) - ref_out).max() <= 2e-2
+    for name, got, ref in (("dq", dq, ref_dq), ("dk", dk, ref_dk), ("dv", dv, ref_dv)):
+        assert np.abs(f(got) - ref).max() <= 2e-2, name
+    assert (f(dk)[0, :70000] == 0).all() and (f(dv)[0, :70000] == 0).all()
