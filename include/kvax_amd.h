@@ -136,8 +136,8 @@ typedef struct kvax_fa_args {
 /* Workspaces (16-byte aligned device memory, contents undefined on entry, reusable right after the
  * call's work on `stream`):
  *   forward:  32 bytes per 64-row kv tile and batch row (tile summaries used to skip dead tiles);
- *   backward: delta [batch, num_heads, q_len] fp32, then the tile summaries of the kv and the
- *             query sequence. */
+ *   backward: delta [batch, num_heads, q_len] fp32, the tile summaries of the kv and the query
+ *             sequence, and the dispatch order of the dK/dV work items (longest first). */
 size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* args);
 size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* args);
 int kvax_fa_fwd(const kvax_fa_args* args, void* workspace, size_t workspace_bytes,

@@ -32,9 +32,38 @@ struct TileSummaryJob {
   void* out;  // int4 [batch, cdiv(len, kTileRows), 2]
   int len;
 };
-int launch_tile_summaries(const TileSummaryJob* jobs, int num_jobs, int batch, hipStream_t stream);
+// `zero` (optional): `batch` int32 counters the kernel clears, for a following launch_tile_order().
+int launch_tile_summaries(const TileSummaryJob* jobs, int num_jobs, int batch, hipStream_t stream,
+                          int32_t* zero = nullptr);
 inline size_t tile_summary_bytes(int batch, int len) {
   return (size_t)batch * cdiv(len, kTileRows) * 32;
 }
+
+
+// Work-item ordering.  A work item is `sub` consecutive tiles of one sequence (the rows one
+// work-group owns); its work is the number of tiles of the other sequence that at least one of its
+// tiles can interact with according to the summaries.  Writes, per batch row, the item indices by
+// decreasing work (ties: lower index first), so that work-groups dispatched in that order finish
+// together instead of leaving the longest items to the end.  One launch; `ws` holds, per batch
+// row, the order (the result, int32 [batch, n_items], at the start), then the work counts and an
+// arrival counter that launch_tile_summaries() must have zeroed (pass `order_counters`).
+struct TileOrderJob {
+  const void* own;   // summaries of the items' sequence, int4 [batch, n_own, 2]
+  const void* opp;   // summaries of the streamed sequence, int4 [batch, n_opp, 2]
+  int32_t* ws;       // tile_order_bytes(batch, n_items)
+  int n_own, n_opp, sub, n_items;
+  int own_is_query;  // the items are query rows or key rows
+};
+int launch_tile_order(const TileOrderJob& job, int batch, hipStream_t stream);
+inline size_t tile_order_bytes(int batch, int n_items) {
+  return ((size_t)batch * (2 * n_items + 1) * sizeof(int32_t) + 15) / 16 * 16;
+}
+inline int32_t* tile_order_counters(int32_t* ws, int batch, int n_items) {
+  return ws + (size_t)batch * 2 * n_items;
+}
+// Below this many items per batch row the dispatch order is left alone (decode, short prompts).
+constexpr int kMinOrderedItems = 16;
+// Above this many the ranking no longer fits the order kernel's LDS (and its cost is quadratic).
+constexpr int kMaxOrderedItems = 8192;
 
 }  // namespace kvax

@@ -60,6 +60,8 @@ struct BwdParams {
   const int4* q_tiles;   // tile summaries [batch, n_q_tiles, 2]
   int n_kv_tiles, n_q_tiles;
   int list_tiles;  // dK/dV kernel: query tiles per chunk of the live-tile bookkeeping
+  int32_t* order_ws;           // room for the dK/dV dispatch order and its scratch
+  const int32_t* dkdv_order;   // kv tiles by decreasing work [batch, tiles], or null
   int flags;
   float scale, scale_log2;
   float scale_log2_abs;  // |scale| * log2(e) > 0, used with K negated when the scale is negative
@@ -120,9 +122,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   int group, rank, g;
   const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, p.group};
   if (!items.decode(blockIdx.x, group, rank, g)) return;
-  const int q_tile = p.num_tiles - 1 - rank;
   const int kv_head = group % p.num_kv_heads;
   const int b = group / p.num_kv_heads;
+  const int q_tile = p.num_tiles - 1 - rank;
   const int head = kv_head * p.group + g;
   const int q0 = q_tile * TQ;
 
@@ -374,12 +376,14 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
   const int pair = wave & 3;
   const bool p_wave = wave < 4;  // role, wave-uniform
 
-  // early kv tiles see the most queries under a causal mask: run them first
-  int group, kv_tile, member;
+  // kv tiles by decreasing work (without an order: early tiles first, which see the most queries
+  // under a causal mask)
+  int group, rank, member;
   const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, 1};
-  if (!items.decode(blockIdx.x, group, kv_tile, member)) return;
+  if (!items.decode(blockIdx.x, group, rank, member)) return;
   const int kv_head = group % p.num_kv_heads;
   const int b = group / p.num_kv_heads;
+  const int kv_tile = p.dkdv_order ? p.dkdv_order[(int64_t)b * p.num_tiles + rank] : rank;
   const int k0 = kv_tile * TKV;
 
   const int kbs = p.bk, qbs = p.bq;
@@ -730,22 +734,38 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   {
     TileSummaryJob jobs[2] = {{p.kv_pos, p.kv_seg, (void*)p.kv_tiles, p.kv_len},
                               {p.q_pos, p.q_seg, (void*)p.q_tiles, p.q_len}};
-    if (int rc = launch_tile_summaries(jobs, 2, p.batch, stream)) return rc;
+    int32_t* counters = tile_order_counters(p.order_ws, p.batch, cdiv(p.kv_len, 128));
+    if (int rc = launch_tile_summaries(jobs, 2, p.batch, stream, counters)) return rc;
   }
   // dQ: two work-groups of four wavefronts per compute unit (each hides the other's prologue,
   // barriers and final stores) when the tile bitmaps fit beside the smaller ring, else one of eight
-  if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
-    static const int cfg = getenv("KVAX_DQ_CFG") ? atoi(getenv("KVAX_DQ_CFG")) : 1;
-    constexpr int kStagesSmall = D == 128 ? 2 : 3;
-    const int small = DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
-    if (cfg == 1 && small <= 80 * 1024) {
+  static const int cfg = getenv("KVAX_DQ_CFG") ? atoi(getenv("KVAX_DQ_CFG")) : 1;
+  constexpr int kStagesSmall = D == 128 ? 2 : 3;
+  const bool run_dq = p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ);
+  const bool run_dkdv = p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV);
+  const bool dq_small =
+      cfg == 1 && DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles) <= 80 * 1024;
+  // dK/dV runs one long work-group per compute unit: dispatch its work items by decreasing number
+  // of live tiles, so that the long ones are not left to the end
+  {
+    static const bool ordered = !(getenv("KVAX_NO_ORDER") && atoi(getenv("KVAX_NO_ORDER")));
+    const int items = cdiv(p.kv_len, 128);
+    if (ordered && run_dkdv && items >= kMinOrderedItems && items <= kMaxOrderedItems) {
+      const TileOrderJob job{p.kv_tiles, p.q_tiles, p.order_ws, p.n_kv_tiles, p.n_q_tiles,
+                             128 / kTileRows, items, 0};
+      if (int rc = launch_tile_order(job, p.batch, stream)) return rc;
+      p.dkdv_order = p.order_ws;
+    }
+  }
+  if (run_dq) {
+    if (dq_small) {
       if (int rc = launch_dq<Tr, D, 4, kStagesSmall>(p, stream)) return rc;
     } else {
       if (int rc = launch_dq<Tr, D, 8, 3>(p, stream)) return rc;
     }
   }
   // dK/dV: 8 wavefronts in 4 role pairs (128 kv rows) per work-group, two per SIMD
-  if (p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV)) {
+  if (run_dkdv) {
     constexpr int NW = 8;
     auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2>;
     static bool done = false;
@@ -775,8 +795,10 @@ static size_t delta_bytes(const kvax_fa_args* a) {
 
 extern "C" size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* a) {
   if (!a || a->batch < 0 || a->q_len < 0 || a->kv_len < 0 || a->num_heads < 0) return 0;
-  // delta [batch, heads, q_len] fp32, then the tile summaries of the kv and query sequences
-  return delta_bytes(a) + tile_summary_bytes(a->batch, a->kv_len) + tile_summary_bytes(a->batch, a->q_len);
+  // delta [batch, heads, q_len] fp32, the tile summaries of the kv and query sequences, and the
+  // dispatch order of the dK/dV work items
+  return delta_bytes(a) + tile_summary_bytes(a->batch, a->kv_len) + tile_summary_bytes(a->batch, a->q_len) +
+         tile_order_bytes(a->batch, cdiv(a->kv_len, 128));
 }
 
 extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
@@ -817,6 +839,7 @@ extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.q_tiles = (const int4*)((char*)workspace + delta_bytes(a) + tile_summary_bytes(a->batch, a->kv_len));
   p.n_kv_tiles = cdiv(a->kv_len, kTileRows);
   p.n_q_tiles = cdiv(a->q_len, kTileRows);
+  p.order_ws = (int32_t*)((char*)p.q_tiles + tile_summary_bytes(a->batch, a->q_len));
   p.q_pos = a->q_pos, p.q_seg = a->q_seg, p.kv_pos = a->kv_pos, p.kv_seg = a->kv_seg;
   for (int i = 0; i < 4; i++) p.dq_mask[i] = a->dq_mask[i], p.dkdv_mask[i] = a->dkdv_mask[i];
   p.q_sb = a->q_strides[0], p.q_ss = a->q_strides[1], p.q_sh = a->q_strides[2];

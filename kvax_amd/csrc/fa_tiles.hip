@@ -16,11 +16,13 @@ namespace {
 
 struct Params {
   TileSummaryJob jobs[2];
+  int32_t* zero;  // one counter per batch row to clear, or null
 };
 
 __global__ __launch_bounds__(256) void tile_summaries_kernel(Params p) {
   const TileSummaryJob& job = p.jobs[blockIdx.z];
   const int lane = threadIdx.x % 64;
+  if (p.zero && blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x == 0) p.zero[blockIdx.y] = 0;
   const int n_tiles = (job.len + kTileRows - 1) / kTileRows;
   const int tile = blockIdx.x * 4 + threadIdx.x / 64;
   if (tile >= n_tiles) return;
@@ -39,11 +41,87 @@ __global__ __launch_bounds__(256) void tile_summaries_kernel(Params p) {
   }
 }
 
+__device__ __forceinline__ const int4* summaries_of(const void* base, int b, int n_tiles) {
+  return reinterpret_cast<const int4*>(base) + 2 * (size_t)b * n_tiles;
+}
+
+// One wavefront per work item counts the opposing tiles the item can interact with; the last
+// work-group of a batch row to finish (arrival counter) then ranks the row's items: the rank of an
+// item is the number of items that go before it.
+__global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int batch) {
+  __shared__ int is_last;
+  const int lane = threadIdx.x % 64;
+  const int item = blockIdx.x * 4 + threadIdx.x / 64;
+  const int b = blockIdx.y;
+  int32_t* order = job.ws + (size_t)b * job.n_items;
+  int32_t* work = job.ws + (size_t)batch * job.n_items + (size_t)b * job.n_items;
+  int32_t* counter = job.ws + (size_t)batch * 2 * job.n_items + b;
+  if (item < job.n_items) {
+    const int4* own = summaries_of(job.own, b, job.n_own);
+    const int4* opp = summaries_of(job.opp, b, job.n_opp);
+    constexpr int kMaxSub = 4;
+    TileParts mine[kMaxSub];
+#pragma unroll
+    for (int s = 0; s < kMaxSub; s++) {
+      const int t = item * job.sub + s;
+      const bool have = s < job.sub && t < job.n_own;
+      mine[s].a = have ? own[2 * t] : empty_summary();
+      mine[s].b = have ? own[2 * t + 1] : empty_summary();
+    }
+    int count = 0;
+    for (int t = lane; t < job.n_opp; t += 64) {
+      TileParts other;
+      other.a = opp[2 * t];
+      other.b = opp[2 * t + 1];
+      bool live = false;
+#pragma unroll
+      for (int s = 0; s < kMaxSub; s++)
+        live |= job.own_is_query ? !parts_cannot_attend(mine[s], other) : !parts_cannot_attend(other, mine[s]);
+      count += live;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) count += __shfl_xor(count, off);
+    if (lane == 0) __hip_atomic_store(work + item, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();  // this work-group's counts are visible before its arrival is
+    is_last = atomicAdd(counter, 1) == (int)gridDim.x - 1;
+  }
+  __syncthreads();
+  if (!is_last) return;
+  __threadfence();
+  extern __shared__ int ranked_work[];  // n_items values, read n_items times each
+  for (int i = threadIdx.x; i < job.n_items; i += 256)
+    ranked_work[i] = __hip_atomic_load(work + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  for (int i = threadIdx.x; i < job.n_items; i += 256) {
+    const int mine = ranked_work[i];
+    int rank = 0;
+    for (int j = 0; j < job.n_items; j++) {
+      const int w = ranked_work[j];
+      rank += (w > mine) | ((w == mine) & (j < i));
+    }
+    order[rank] = i;
+  }
+}
+
 }  // namespace
 
-int launch_tile_summaries(const TileSummaryJob* jobs, int num_jobs, int batch, hipStream_t stream) {
+int launch_tile_order(const TileOrderJob& job, int batch, hipStream_t stream) {
+  if (job.sub < 1 || job.sub > 4) return fail(KVAX_EINVAL, "work items of %d tiles", job.sub);
+  if (job.n_items > kMaxOrderedItems) return fail(KVAX_EINVAL, "%d work items to order", job.n_items);
+  if (job.n_items == 0 || batch == 0) return KVAX_OK;
+  hipLaunchKernelGGL(tile_order_kernel, dim3(cdiv(job.n_items, 4), batch), dim3(256),
+                     job.n_items * sizeof(int), stream, job, batch);
+  return check_launch("tile_order_kernel");
+}
+
+int launch_tile_summaries(const TileSummaryJob* jobs, int num_jobs, int batch, hipStream_t stream,
+                          int32_t* zero) {
   static_assert(kTileRows == 64, "one lane per row");
   Params p{};
+  p.zero = zero;
   int max_tiles = 0;
   for (int i = 0; i < num_jobs; i++) {
     p.jobs[i] = jobs[i];
