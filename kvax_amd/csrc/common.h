@@ -42,11 +42,12 @@ inline size_t tile_summary_bytes(int batch, int len) {
 
 // Work-item ordering.  A work item is `sub` consecutive tiles of one sequence (the rows one
 // work-group owns); its work is the number of tiles of the other sequence that at least one of its
-// tiles can interact with according to the summaries.  Writes, per batch row, the item indices by
-// decreasing work (ties: lower index first), so that work-groups dispatched in that order finish
-// together instead of leaving the longest items to the end.  One launch; `ws` holds, per batch
-// row, the order (the result, int32 [batch, n_items], at the start), then the work counts and an
-// arrival counter that launch_tile_summaries() must have zeroed (pass `order_counters`).
+// tiles can interact with according to the summaries.  Writes, per batch row, the dispatch order of
+// the items: those with more than the row's mean work in index order, then the others by decreasing
+// work (ties: lower index first), so that the launch ends on short items.  One launch; `ws` holds
+// the order (the result, int32 [batch, n_items], at the start), then the work counts and one
+// arrival counter per batch row, which launch_tile_summaries() must have zeroed (pass it
+// tile_order_counters(ws, ...)).
 struct TileOrderJob {
   const void* own;   // summaries of the items' sequence, int4 [batch, n_own, 2]
   const void* opp;   // summaries of the streamed sequence, int4 [batch, n_opp, 2]

@@ -61,7 +61,7 @@ struct BwdParams {
   int n_kv_tiles, n_q_tiles;
   int list_tiles;  // dK/dV kernel: query tiles per chunk of the live-tile bookkeeping
   int32_t* order_ws;           // room for the dK/dV dispatch order and its scratch
-  const int32_t* dkdv_order;   // kv tiles by decreasing work [batch, tiles], or null
+  const int32_t* dkdv_order;   // dispatch order of the kv tiles [batch, tiles], or null
   int flags;
   float scale, scale_log2;
   float scale_log2_abs;  // |scale| * log2(e) > 0, used with K negated when the scale is negative
@@ -376,8 +376,8 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
   const int pair = wave & 3;
   const bool p_wave = wave < 4;  // role, wave-uniform
 
-  // kv tiles by decreasing work (without an order: early tiles first, which see the most queries
-  // under a causal mask)
+  // kv tiles in the computed dispatch order (without one: early tiles first, which see the most
+  // queries under a causal mask)
   int group, rank, member;
   const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, 1};
   if (!items.decode(blockIdx.x, group, rank, member)) return;
@@ -739,18 +739,16 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   }
   // dQ: two work-groups of four wavefronts per compute unit (each hides the other's prologue,
   // barriers and final stores) when the tile bitmaps fit beside the smaller ring, else one of eight
-  static const int cfg = getenv("KVAX_DQ_CFG") ? atoi(getenv("KVAX_DQ_CFG")) : 1;
   constexpr int kStagesSmall = D == 128 ? 2 : 3;
   const bool run_dq = p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ);
   const bool run_dkdv = p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV);
   const bool dq_small =
-      cfg == 1 && DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles) <= 80 * 1024;
-  // dK/dV runs one long work-group per compute unit: dispatch its work items by decreasing number
-  // of live tiles, so that the long ones are not left to the end
+      DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles) <= 80 * 1024;
+  // dK/dV runs one long work-group per compute unit: its light work items are dispatched last, by
+  // decreasing number of live tiles, so that the launch does not end on a few long ones
   {
-    static const bool ordered = !(getenv("KVAX_NO_ORDER") && atoi(getenv("KVAX_NO_ORDER")));
     const int items = cdiv(p.kv_len, 128);
-    if (ordered && run_dkdv && items >= kMinOrderedItems && items <= kMaxOrderedItems) {
+    if (run_dkdv && items >= kMinOrderedItems && items <= kMaxOrderedItems) {
       const TileOrderJob job{p.kv_tiles, p.q_tiles, p.order_ws, p.n_kv_tiles, p.n_q_tiles,
                              128 / kTileRows, items, 0};
       if (int rc = launch_tile_order(job, p.batch, stream)) return rc;

@@ -379,10 +379,10 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
 // and final stores) whenever the tile bitmaps of the sequence fit beside the smaller ring;
 // otherwise one work-group of eight wavefronts.
 template <class Tr, int D>
-int launch_fwd_auto(const FwdParams& p, hipStream_t stream, int cfg) {
+int launch_fwd_auto(const FwdParams& p, hipStream_t stream) {
   constexpr int kStagesSmall = D == 128 ? 2 : 3;
   const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
-  if (cfg == 1 && small <= 80 * 1024) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
+  if (small <= 80 * 1024) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
   return launch_fwd<Tr, D, 1, 8, 2, 3>(p, stream);
 }
 
@@ -473,8 +473,7 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
   const bool bf16 = a->dtype == KVAX_BF16;
-  static const int cfg = getenv("KVAX_FWD_CFG") ? atoi(getenv("KVAX_FWD_CFG")) : 1;
   if (a->head_dim == 128)
-    return bf16 ? launch_fwd_auto<Bf16, 128>(p, stream, cfg) : launch_fwd_auto<F16, 128>(p, stream, cfg);
-  return bf16 ? launch_fwd_auto<Bf16, 64>(p, stream, cfg) : launch_fwd_auto<F16, 64>(p, stream, cfg);
+    return bf16 ? launch_fwd_auto<Bf16, 128>(p, stream) : launch_fwd_auto<F16, 128>(p, stream);
+  return bf16 ? launch_fwd_auto<Bf16, 64>(p, stream) : launch_fwd_auto<F16, 64>(p, stream);
 }

@@ -69,6 +69,7 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
       mine[s].b = have ? own[2 * t + 1] : empty_summary();
     }
     int count = 0;
+#pragma unroll 4
     for (int t = lane; t < job.n_opp; t += 64) {
       TileParts other;
       other.a = opp[2 * t];
@@ -91,16 +92,30 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
   __syncthreads();
   if (!is_last) return;
   __threadfence();
-  extern __shared__ int ranked_work[];  // n_items values, read n_items times each
-  for (int i = threadIdx.x; i < job.n_items; i += 256)
-    ranked_work[i] = __hip_atomic_load(work + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  // Heavy items (work above the row's mean) keep their index order: neighbours stream the same
+  // tiles of the other sequence at about the same time, which is what keeps those tiles in L2, and
+  // they carry most of the traffic.  Light items follow by decreasing work and fill the gaps at the
+  // end of the launch.
+  extern __shared__ int item_work[];  // n_items values
+  __shared__ int total;
+  if (threadIdx.x == 0) total = 0;
   __syncthreads();
+  int part = 0;
   for (int i = threadIdx.x; i < job.n_items; i += 256) {
-    const int mine = ranked_work[i];
+    item_work[i] = __hip_atomic_load(work + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    part += item_work[i];
+  }
+  atomicAdd(&total, part);
+  __syncthreads();
+  const int light_max = total / job.n_items;  // work <= this: light
+  for (int i = threadIdx.x; i < job.n_items; i += 256) {
+    const int mine = item_work[i];
+    const bool light = mine <= light_max;
     int rank = 0;
     for (int j = 0; j < job.n_items; j++) {
-      const int w = ranked_work[j];
-      rank += (w > mine) | ((w == mine) & (j < i));
+      const int w = item_work[j];
+      const bool w_light = w <= light_max;
+      rank += light ? (!w_light | (w > mine) | ((w == mine) & (j < i))) : (!w_light & (j < i));
     }
     order[rank] = i;
   }
