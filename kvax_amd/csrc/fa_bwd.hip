@@ -748,7 +748,8 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   // decreasing number of live tiles, so that the launch does not end on a few long ones
   {
     const int items = cdiv(p.kv_len, 128);
-    if (run_dkdv && items >= kMinOrderedItems && items <= kMaxOrderedItems) {
+    if (run_dkdv && items >= kMinOrderedItems && items <= kMaxOrderedItems &&
+        (int64_t)items * (p.n_q_tiles + 2) < 0x7fffffff) {
       const TileOrderJob job{p.kv_tiles, p.q_tiles, p.order_ws, p.n_kv_tiles, p.n_q_tiles,
                              128 / kTileRows, items, 0};
       if (int rc = launch_tile_order(job, p.batch, stream)) return rc;

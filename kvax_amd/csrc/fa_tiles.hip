@@ -96,26 +96,37 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
   // tiles of the other sequence at about the same time, which is what keeps those tiles in L2, and
   // they carry most of the traffic.  Light items follow by decreasing work and fill the gaps at the
   // end of the launch.
-  extern __shared__ int item_work[];  // n_items values
+  // Both rules in one sort key (unique per item): heavy items index, light items
+  // n * (1 + max work - work) + index; the rank of an item is the number of smaller keys.
+  extern __shared__ __attribute__((aligned(16))) int keys[];  // n_items values, padded to a multiple of 4
   __shared__ int total;
   if (threadIdx.x == 0) total = 0;
   __syncthreads();
   int part = 0;
   for (int i = threadIdx.x; i < job.n_items; i += 256) {
-    item_work[i] = __hip_atomic_load(work + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    part += item_work[i];
+    keys[i] = __hip_atomic_load(work + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    part += keys[i];
   }
-  atomicAdd(&total, part);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off);
+  if (lane == 0) atomicAdd(&total, part);
   __syncthreads();
   const int light_max = total / job.n_items;  // work <= this: light
+  const int padded = (job.n_items + 3) & ~3;
+  for (int i = threadIdx.x; i < padded; i += 256) {
+    const int w = i < job.n_items ? keys[i] : 0;
+    int key = 0x7fffffff;  // padding: larger than every real key
+    if (i < job.n_items) key = w > light_max ? i : job.n_items * (1 + job.n_opp - w) + i;
+    keys[i] = key;  // same thread read keys[i] above
+  }
+  __syncthreads();
   for (int i = threadIdx.x; i < job.n_items; i += 256) {
-    const int mine = item_work[i];
-    const bool light = mine <= light_max;
+    const int mine = keys[i];
     int rank = 0;
-    for (int j = 0; j < job.n_items; j++) {
-      const int w = item_work[j];
-      const bool w_light = w <= light_max;
-      rank += light ? (!w_light | (w > mine) | ((w == mine) & (j < i))) : (!w_light & (j < i));
+#pragma unroll 4
+    for (int j = 0; j < padded; j += 4) {
+      const int4 k = *reinterpret_cast<const int4*>(keys + j);
+      rank += (k.x < mine) + (k.y < mine) + (k.z < mine) + (k.w < mine);
     }
     order[rank] = i;
   }
@@ -125,10 +136,12 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
 
 int launch_tile_order(const TileOrderJob& job, int batch, hipStream_t stream) {
   if (job.sub < 1 || job.sub > 4) return fail(KVAX_EINVAL, "work items of %d tiles", job.sub);
-  if (job.n_items > kMaxOrderedItems) return fail(KVAX_EINVAL, "%d work items to order", job.n_items);
+  // the sort keys must fit 31 bits
+  if (job.n_items > kMaxOrderedItems || (int64_t)job.n_items * (job.n_opp + 2) >= 0x7fffffff)
+    return fail(KVAX_EINVAL, "%d work items over %d tiles to order", job.n_items, job.n_opp);
   if (job.n_items == 0 || batch == 0) return KVAX_OK;
   hipLaunchKernelGGL(tile_order_kernel, dim3(cdiv(job.n_items, 4), batch), dim3(256),
-                     job.n_items * sizeof(int), stream, job, batch);
+                     (job.n_items + 3) / 4 * 4 * sizeof(int), stream, job, batch);
   return check_launch("tile_order_kernel");
 }
 
