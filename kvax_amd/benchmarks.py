@@ -77,8 +77,6 @@ def report(name: str, seconds: float, tflops_reference_model: float, tflops_unma
 
 def make_inputs(batch_size, query_seq_len, kv_seq_len, num_heads, num_kv_heads, qk_head_dim,
                 value_head_dim, num_segments, num_pad_tokens, device):
-    if qk_head_dim != value_head_dim:
-        raise click.UsageError("the kernels need --qk-head-dim equal to --value-head-dim")
     return make_random_attention_inputs(
         batch_size=batch_size, query_seq_len=query_seq_len, kv_seq_len=kv_seq_len,
         num_query_heads=num_heads, num_kv_heads=num_kv_heads, qk_head_dim=qk_head_dim,
@@ -117,7 +115,7 @@ def run_kvax(data, scale, specs, mesh, *, backward, assume_sequential_positions,
     original token order plus the two TFLOP figures per iteration."""
     query, key, value, q_pos, q_seg, kv_pos, kv_seg = data
     batch, q_len, heads, dim = query.shape
-    kv_len = key.shape[1]
+    kv_len, dim_v = key.shape[1], value.shape[3]
     fwd_params = get_default_flash_attention_params(backward=False)
     bwd_params = get_default_flash_attention_params(backward=True)
     device = query.device
@@ -166,10 +164,10 @@ def run_kvax(data, scale, specs, mesh, *, backward, assume_sequential_positions,
 
     density = calculate_mask_sparsity(mask[0], fwd_params.query_block_size,
                                       fwd_params.kv_block_size, q_len, kv_len)
-    dense = get_multi_head_attention_tflops(batch, q_len, kv_len, heads, dim, dim, causal=False,
+    dense = get_multi_head_attention_tflops(batch, q_len, kv_len, heads, dim, dim_v, causal=False,
                                             forward_pass=True, backward_pass=backward)
     pairs = count_unmasked_pairs(*(t.cpu().numpy() for t in data[3:]))
-    exact = attention_tflops_from_pairs(pairs, heads, dim, dim, True, backward)
+    exact = attention_tflops_from_pairs(pairs, heads, dim, dim_v, True, backward)
     report(name, seconds, dense * density, exact)
     return zero_padding_rows(out, data[4]), grads
 
@@ -218,7 +216,8 @@ def single_device_benchmark(backward: bool, *, num_iters, batch_size, query_seq_
     device = device_or_fail()
     data, scale = make_inputs(batch_size, query_seq_len, kv_seq_len, num_heads, num_kv_heads,
                               qk_head_dim, value_head_dim, num_segments, num_pad_tokens, device)
-    dout = torch.randn_like(data[0]) if backward else None
+    dout = torch.randn(data[0].shape[:3] + data[2].shape[3:], dtype=data[0].dtype, device=device) \
+        if backward else None
     out, grads = run_kvax(
         data, scale, TP_SPECS, Mesh({"data": 1, "model": 1}), backward=backward,
         assume_sequential_positions=assume_sequential_positions, permute=False,
@@ -244,7 +243,8 @@ def context_parallel_benchmark(backward: bool, *, num_iters, batch_size, query_s
     device = device_or_fail()
     data, scale = make_inputs(batch_size, query_seq_len, kv_seq_len, num_heads, num_kv_heads,
                               qk_head_dim, value_head_dim, num_segments, 0, device)
-    dout = torch.randn_like(data[0]) if backward else None
+    dout = torch.randn(data[0].shape[:3] + data[2].shape[3:], dtype=data[0].dtype, device=device) \
+        if backward else None
     shared = dict(backward=backward, assume_sequential_positions=assume_sequential_positions,
                   show_attention_mask=show_attention_mask, num_iters=num_iters, dout=dout)
     cp = run_kvax(data, scale, CP_SPECS, Mesh({"data": 1, "context": context_parallel_degree}),

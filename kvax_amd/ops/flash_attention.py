@@ -29,7 +29,10 @@ from kvax_amd.utils.sharding import context_parallel_degree
 from kvax_amd.utils.specs import get_attention_specs
 from kvax_amd.utils.typing import AttentionMask, DeviceArray
 
-SUPPORTED_HEAD_DIMS = (64, 128)
+SUPPORTED_HEAD_DIMS = (64, 128)  # what the kernels are built for
+# What ``flash_attention`` takes for query/key (the reference's list, flash_attention_triton.py:1397,
+# up to the largest built size); smaller ones and a different value head_dim are zero-padded.
+ACCEPTED_HEAD_DIMS = (16, 32, 64, 128)
 _DTYPES = {torch.bfloat16: _native.KVAX_BF16, torch.float16: _native.KVAX_F16}
 
 
@@ -67,12 +70,15 @@ def _check_inputs(query, key, value):
         raise TypeError("query, key and value must share one dtype")
     b, sq, hq, d = query.shape
     bk, sk, hkv, dk_ = key.shape
-    if value.shape != key.shape:
-        raise ValueError(f"key {tuple(key.shape)} and value {tuple(value.shape)} must match")
+    if value.shape[:3] != key.shape[:3]:
+        raise ValueError(f"key {tuple(key.shape)} and value {tuple(value.shape)} must match "
+                         "in batch, length and heads")
     if bk != b or dk_ != d:
         raise ValueError("query and key/value disagree on batch size or head_dim")
-    if d not in SUPPORTED_HEAD_DIMS:
-        raise ValueError(f"Attention hid_dim can take values {list(SUPPORTED_HEAD_DIMS)}")
+    if d not in ACCEPTED_HEAD_DIMS:
+        raise ValueError(f"Attention hid_dim can take values {list(ACCEPTED_HEAD_DIMS)}")
+    if not 1 <= value.shape[3] <= SUPPORTED_HEAD_DIMS[-1]:
+        raise ValueError(f"value head_dim {value.shape[3]} is outside 1..{SUPPORTED_HEAD_DIMS[-1]}")
     if hq % hkv != 0:
         raise ValueError(f"num_heads {hq} must be divisible by num_kv_heads {hkv}")
 
@@ -256,6 +262,8 @@ def flash_attention(
     """Attention over packed documents with a block-sparse mask.
 
     Arguments and defaults as in the reference (flash_attention_triton.py:2027-2095).
+    Query/key head dims 16, 32, 64, 128 and any value head dim up to 128 are taken (the kernels run
+    at 64 or 128; other sizes are zero-padded here).
     ``memory_optimized_gqa_backward`` is accepted and has no effect: dK/dV are always reduced
     over the query heads of a group inside the kernel, which is what the flag asks for.
     ``debug`` is accepted and ignored.  With ``assume_sequential_positions`` the causal test uses
@@ -282,9 +290,20 @@ def flash_attention(
     if assume_sequential_positions:
         query_positions, kv_positions = _sequential_positions(
             query, key, cp, permute_tokens_for_load_balance)
-    return _FlashAttentionFn.apply(
+    # Head dims the kernels are not built for: zero columns change neither Q K^T nor the real
+    # columns of P V, so the tensors are padded to the next built size and the output is cut back
+    # (autograd does the same to the gradients).
+    d_qk, d_v = query.shape[3], value.shape[3]
+    d_run = next(d for d in SUPPORTED_HEAD_DIMS if d >= max(d_qk, d_v))
+    if d_qk != d_run:
+        query = torch.nn.functional.pad(query, (0, d_run - d_qk))
+        key = torch.nn.functional.pad(key, (0, d_run - d_qk))
+    if d_v != d_run:
+        value = torch.nn.functional.pad(value, (0, d_run - d_v))
+    out = _FlashAttentionFn.apply(
         query, key, value, query_positions, query_segment_ids, kv_positions, kv_segment_ids,
         tuple(mask), float(scale), fwd_params, bwd_params, cp)
+    return out if d_v == d_run else out[..., :d_v]
 
 
 def _sequential_positions(query, key, cp: int, permuted: bool):

@@ -102,6 +102,22 @@ def test_backward_matches_dense_oracle(device, case):
     check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if hkv == 1 else ATOL)
 
 
+@pytest.mark.parametrize("d_qk, d_v, hq, hkv", [(16, 16, 8, 8), (32, 32, 8, 2), (32, 96, 4, 2),
+                                               (128, 64, 4, 4), (64, 40, 4, 1)])
+def test_backward_small_and_unequal_head_dims(device, d_qk, d_v, hq, hkv):
+    """Head dims below the built sizes and value dims that differ from the qk one go through zero
+    padding in the wrapper; the gradients come back in the callers' shapes."""
+    data, scale = make_random_attention_inputs(2, 384, 384, hq, hkv, d_qk, d_v, seed=d_qk + d_v,
+                                               num_pad_tokens=60,
+                                               list_of_segment_lengths=[100, 150, -1], device=device)
+    dout = torch.randn((2, 384, hq, d_v), generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).to(device)
+    out, dq, dk, dv = run_backward(data, scale, (64, 64), (64, 64), dout)
+    assert out.shape == dout.shape and dq.shape == data[0].shape
+    assert dk.shape == data[1].shape and dv.shape == data[2].shape
+    refs = oracle_backward(data, scale, dout)
+    check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if hkv == 1 else ATOL)
+
+
 @pytest.mark.parametrize("case", [CASES[7], CASES[6], CASES[8]])
 def test_fp32_dkdv_within_plain_bound(device, case):
     """dK/dV straight from the fp32 accumulators: plain max abs error <= 2e-2, no relative term."""

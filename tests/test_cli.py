@@ -29,6 +29,12 @@ def test_single_device_commands(device, caplog, command, sequential):
 
 
 @pytest.mark.gpu
+def test_head_dims_of_the_reference_tests(device, caplog):
+    text = _invoke(["mha_bwd", *SMALL, "--qk-head-dim", "16", "--value-head-dim", "32"], caplog)
+    assert "outputs agree with the library attention" in text
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("command", ["mha_cp", "mha_cp_bwd"])
 @pytest.mark.parametrize("permute", ["True", "False"])
 def test_context_parallel_commands(device, caplog, command, permute):

@@ -86,6 +86,34 @@ def test_forward_matches_dense_oracle(device, case, dtype):
     check(out, oracle_forward(data, scale), data[4])
 
 
+# The reference's own forward cases run at head_dim 16 (tests/test_attention.py:308-340): taken
+# through zero padding to the built sizes, as are value head dims that differ from the qk one.
+@pytest.mark.parametrize("sq, sk, hq, hkv, d_qk, d_v, pad", [
+    (384, 384, 8, 8, 16, 16, 0), (400, 300, 8, 8, 16, 16, 0), (1, 256, 8, 8, 16, 16, 0),
+    (256, 1, 8, 8, 16, 16, 0), (1, 3, 8, 8, 16, 16, 0), (384, 384, 16, 8, 16, 16, 383),
+    (384, 384, 16, 1, 16, 16, 100), (384, 384, 8, 4, 32, 32, 50), (384, 384, 8, 4, 32, 96, 50),
+    (256, 320, 4, 2, 128, 64, 0), (256, 320, 4, 2, 64, 8, 17),
+])
+def test_forward_small_and_unequal_head_dims(device, sq, sk, hq, hkv, d_qk, d_v, pad):
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d_qk, d_v, seed=sq + sk + d_qk + d_v,
+                                               num_pad_tokens=min(pad, sk - 1), device=device)
+    out = run_forward(data, scale, 64, 64)
+    assert out.shape == (2, sq, hq, d_v)
+    check(out, oracle_forward(data, scale), data[4])
+
+
+def test_head_dims_that_are_not_taken(device):
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 256, 256, device=device)
+    with pytest.raises(ValueError, match="hid_dim"):
+        run_forward(data, scale, 64, 64)
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 24, 24, device=device)
+    with pytest.raises(ValueError, match="hid_dim"):
+        run_forward(data, scale, 64, 64)
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 64, 192, device=device)
+    with pytest.raises(ValueError, match="value head_dim"):
+        run_forward(data, scale, 64, 64)
+
+
 def test_forward_fp16(device):
     data, scale = make_random_attention_inputs(1, 512, 512, 4, 2, 128, 128, seed=3,
                                                num_pad_tokens=50, dtype=torch.float16, device=device)
