@@ -82,13 +82,13 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) count += __shfl_xor(count, off);
-    if (lane == 0) __hip_atomic_store(work + item, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) {
+      __hip_atomic_store(work + item, count, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __threadfence();  // the count is visible device-wide before this work-group's arrival is
+    }
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    __threadfence();  // this work-group's counts are visible before its arrival is
-    is_last = atomicAdd(counter, 1) == (int)gridDim.x - 1;
-  }
+  if (threadIdx.x == 0) is_last = atomicAdd(counter, 1) == (int)gridDim.x - 1;
   __syncthreads();
   if (!is_last) return;
   __threadfence();

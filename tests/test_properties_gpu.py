@@ -111,10 +111,10 @@ def test_single_token_sequence(device):
     assert torch.equal(dv.float(), torch.full_like(dv.float(), 2.0))
 
 
-@pytest.mark.parametrize("q_len, kv_len", [(0, 64), (64, 0), (0, 0)])
+@pytest.mark.parametrize("q_len, kv_len", [(0, 64), (64, 0), (0, 0), (0, 4096), (4096, 0)])
 def test_empty_sequences(device, q_len, kv_len):
-    q = torch.zeros(1, q_len, 4, 64, dtype=torch.bfloat16, device=device)
-    k = torch.zeros(1, kv_len, 2, 64, dtype=torch.bfloat16, device=device)
+    q = torch.ones(1, q_len, 4, 64, dtype=torch.bfloat16, device=device)
+    k = torch.ones(1, kv_len, 2, 64, dtype=torch.bfloat16, device=device)
     ids = [torch.zeros(1, n, dtype=torch.int32, device=device) for n in (q_len, q_len, kv_len, kv_len)]
     out, dq, dk, dv = _run((q, k, k.clone(), *ids), 0.125)
     assert out.shape == q.shape and dq.shape == q.shape and dk.shape == k.shape
