@@ -44,12 +44,18 @@ struct FwdParams {
   int64_t v_sb, v_ss, v_sh;
   int64_t o_sb, o_ss, o_sh;
   int batch, q_len, kv_len, num_heads, num_kv_heads, group;
+  bool split_mode;
   int qbs, kbs, n_qblocks;
   int num_q_tiles, total_items;
   const int4* kv_tiles;  // tile summaries [batch, n_kv_tiles]
   int n_kv_tiles;
   uint32_t q_sign;       // 0x80008000 when the scale is negative: Q is negated on load
   float scale_log2;      // |scale| * log2(e), > 0
+  // split mode (short query sequences, see fa_fwd_kernel): rows are (query, head of the group)
+  // pairs; each work-group takes 1 / num_splits of the live kv tiles and leaves a partial result
+  int num_splits, part_rows;  // rows per tile that have a partial (<= TQ)
+  float* part_o;              // [items, num_splits, part_rows, D] unnormalised O
+  float* part_ml;             // [items, num_splits, part_rows, 2] running max (base 2) and sum
 };
 
 template <int D, int STAGES>
@@ -62,7 +68,13 @@ struct FwdSmem {
 
 // One work-group: NW wavefronts x (32 * MQ) query rows of one (batch, head); streams the live kv
 // tiles through a STAGES-deep ring of LDS stages filled by asynchronous copies.
-template <class Tr, int D, int MQ, int NW, int WPS, int STAGES>
+//
+// SPLIT (short query sequences, e.g. decoding one token against a long key sequence, where one
+// work-group per (batch, head) would leave most of the chip idle and read the keys serially): the
+// rows of a work-group are (query, query head) pairs of one (batch, kv head) - all heads of a GQA
+// group share the key tiles they stream - and the live kv tiles are divided over num_splits
+// work-groups, each leaving an unnormalised partial result that fa_fwd_combine_kernel merges.
+template <class Tr, int D, int MQ, int NW, int WPS, int STAGES, bool SPLIT>
 __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p) {
   using vec8 = typename Tr::vec8;
   using Smem = FwdSmem<D, STAGES>;
@@ -79,14 +91,23 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   const int c = lane % 32, h = lane / 32;
 
   // ---- work item: heads of a GQA group adjacent, long (late) query tiles first -------------
-  int group, rank, g;
-  const ItemMap items{p.batch * p.num_kv_heads, p.num_q_tiles, p.group};
-  if (!items.decode(blockIdx.x, group, rank, g)) return;
+  int group, rank, g = 0, split = 0, item = 0;
+  if (SPLIT) {
+    static_assert(!SPLIT || MQ == 1, "split mode maps one row per lane");
+    split = blockIdx.x % p.num_splits;
+    item = blockIdx.x / p.num_splits;
+    rank = p.num_q_tiles - 1 - item % p.num_q_tiles;
+    group = item / p.num_q_tiles;
+  } else {
+    const ItemMap items{p.batch * p.num_kv_heads, p.num_q_tiles, p.group};
+    if (!items.decode(blockIdx.x, group, rank, g)) return;
+  }
   const int q_tile = p.num_q_tiles - 1 - rank;
   const int kv_head = group % p.num_kv_heads;
   const int b = group / p.num_kv_heads;
-  const int head = kv_head * p.group + g;
-  const int q0 = q_tile * TQ;
+  const int head = kv_head * p.group + g;  // split mode: first head of the group
+  const int q0 = q_tile * TQ;              // split mode: in (query, head) pairs
+  const int rows_total = SPLIT ? p.q_len * p.group : p.q_len;
 
   const int32_t* q_seg = p.q_seg + (int64_t)b * p.q_len;
   const int32_t* q_pos = p.q_pos + (int64_t)b * p.q_len;
@@ -102,8 +123,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   // query blocks it covers, intersection of the full ranges (element units) ---------------------
   int lo = 0x7fffffff, hi = 0, flo = 0, fhi = 0x7fffffff;
   {
-    const int qb0 = q0 / p.qbs;
-    const int qb1 = min((q0 + TQ - 1) / p.qbs, p.n_qblocks - 1);
+    const int qb0 = (SPLIT ? q0 / p.group : q0) / p.qbs;
+    const int qb1 = min((SPLIT ? (q0 + TQ - 1) / p.group : q0 + TQ - 1) / p.qbs, p.n_qblocks - 1);
     for (int qb = qb0; qb <= qb1; qb++) {
       const int64_t mi = (int64_t)b * p.n_qblocks + qb;
       const int l_ = p.lower[mi] * p.kbs, u_ = p.upper[mi] * p.kbs;
@@ -121,13 +142,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   const int tf_lo = (flo + kTK - 1) / kTK, tf_hi = fhi / kTK;
 
   // ---- per-lane query columns ------------------------------------------------------------
-  int qrow[MQ], qseg[MQ], qpos[MQ], col_lo[MQ];
+  // qrow: the lane's query index; lane_head: its query head (split mode: per lane)
+  int qrow[MQ], lane_head[MQ], qseg[MQ], qpos[MQ], col_lo[MQ];
+  bool row_in[MQ];
   unsigned col_width[MQ];
   TileParts mine[MQ];
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
-    qrow[qt] = q0 + (wave * MQ + qt) * 32 + c;
-    const bool in = qrow[qt] < p.q_len;
+    const int row = q0 + (wave * MQ + qt) * 32 + c;
+    row_in[qt] = row < rows_total;
+    qrow[qt] = SPLIT ? row / p.group : row;
+    lane_head[qt] = SPLIT ? head + row % p.group : head;
+    const bool in = row_in[qt];
     qseg[qt] = in ? q_seg[qrow[qt]] : -1;
     qpos[qt] = in ? q_pos[qrow[qt]] : 0;
     col_lo[qt] = 0;
@@ -156,6 +182,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
   __syncthreads();
   const int n_live = *live_count;
+  // this work-group's share of the live tiles
+  const int i_lo = SPLIT ? (int)((int64_t)n_live * split / p.num_splits) : 0;
+  const int i_hi = SPLIT ? (int)((int64_t)n_live * (split + 1) / p.num_splits) : n_live;
 
   f32x16 o[DT][MQ];
   float m_run[MQ], l_run[MQ];
@@ -169,14 +198,15 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       for (int i = 0; i < 16; i++) o[dt][qt][i] = 0.f;
   }
 
-  if (n_live > 0) {
+  if (i_hi > i_lo) {
     // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step.
     // A negative scale is folded into Q so that the softmax below can assume scale_log2 > 0.
     vec8 qf[MQ][KSTEPS];
 #pragma unroll
     for (int qt = 0; qt < MQ; qt++) {
-      const bool in = qrow[qt] < p.q_len;
-      const char* row = qbase + (int64_t)(in ? qrow[qt] : 0) * p.q_ss * 2;
+      const bool in = row_in[qt];
+      const char* row = (SPLIT ? p.q + ((int64_t)b * p.q_sb + (int64_t)lane_head[qt] * p.q_sh) * 2 : qbase) +
+                        (int64_t)(in ? qrow[qt] : 0) * p.q_ss * 2;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ks++) {
         uint4 u = make_uint4(0, 0, 0, 0);
@@ -209,22 +239,22 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     };
 
     // entries of the live list for iterations i, i + 1, i + 2 (read ahead of their use)
-    uint32_t e0 = live_list[0];
-    uint32_t e1 = n_live > 1 ? live_list[1] : 0;
-    uint32_t e2 = n_live > 2 ? live_list[2] : 0;
+    uint32_t e0 = live_list[i_lo];
+    uint32_t e1 = i_lo + 1 < i_hi ? live_list[i_lo + 1] : 0;
+    uint32_t e2 = i_lo + 2 < i_hi ? live_list[i_lo + 2] : 0;
     issue(e0 & 0xffffff, 0);
-    if (STAGES == 3 && n_live > 1) issue(e1 & 0xffffff, 1);
+    if (STAGES == 3 && i_lo + 1 < i_hi) issue(e1 & 0xffffff, 1);
 
     int stage = 0;
-    for (int i = 0; i < n_live; i++) {
+    for (int i = i_lo; i < i_hi; i++) {
       // tile i has landed once at most the copies of tile i + 1 are outstanding
-      if (STAGES == 3 && i + 1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      if (STAGES == 3 && i + 1 < i_hi) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       __syncthreads();
-      const uint32_t e3 = i + 3 < n_live ? live_list[i + 3] : 0;
+      const uint32_t e3 = i + 3 < i_hi ? live_list[i + 3] : 0;
       if (STAGES == 3) {
-        if (i + 2 < n_live) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
+        if (i + 2 < i_hi) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
       } else {
-        if (i + 1 < n_live) issue(e1 & 0xffffff, stage ^ 1);
+        if (i + 1 < i_hi) issue(e1 & 0xffffff, stage ^ 1);
       }
       const int t = e0 & 0xffffff;
 
@@ -328,14 +358,33 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     }
   }
 
+  // ---- split mode with several splits: leave the unnormalised partial result ---------------
+  if (SPLIT && p.num_splits > 1) {
+    const int prow = wave * 32 + c;  // MQ == 1
+    if (row_in[0] && prow < p.part_rows) {
+      const int64_t slot = ((int64_t)item * p.num_splits + split) * p.part_rows + prow;
+      float* po = p.part_o + slot * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++)
+          *reinterpret_cast<float4*>(po + 32 * dt + 8 * g4 + 4 * h) =
+              make_float4(o[dt][0][4 * g4 + 0], o[dt][0][4 * g4 + 1], o[dt][0][4 * g4 + 2], o[dt][0][4 * g4 + 3]);
+      const float l = l_run[0] + xor32(l_run[0]);
+      if (h == 0) *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], l);
+    }
+    return;
+  }
+
   // ---- epilogue: normalise, write O (query dtype) and lse --------------------------------
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
     const float l = l_run[qt] + xor32(l_run[qt]);
     const bool alive = l > 0.f && col_width[qt] > 0;  // padding / out-of-range rows stay zero
     const float inv = alive ? 1.f / l : 0.f;
-    if (qrow[qt] < p.q_len) {
-      char* row = obase + (int64_t)qrow[qt] * p.o_ss * 2;
+    if (row_in[qt]) {
+      char* row = (SPLIT ? p.out + ((int64_t)b * p.o_sb + (int64_t)lane_head[qt] * p.o_sh) * 2 : obase) +
+                  (int64_t)qrow[qt] * p.o_ss * 2;
 #pragma unroll
       for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -345,19 +394,98 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           u.y = Tr::pack2(o[dt][qt][4 * g4 + 2] * inv, o[dt][qt][4 * g4 + 3] * inv);
           *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
         }
-      if (h == 0) lse[qrow[qt]] = alive ? m_run[qt] + fast_log2(l) : 0.f;
+      if (h == 0)
+        (SPLIT ? p.lse + ((int64_t)b * p.num_heads + lane_head[qt]) * p.q_len : lse)[qrow[qt]] =
+            alive ? m_run[qt] + fast_log2(l) : 0.f;
     }
   }
 }
 
-template <class Tr, int D, int MQ, int NW, int WPS, int STAGES = 3>
+// Merges the partial results of the split mode: one work-group per (item, row), one thread per
+// head-dim element.  M = max m_s, L = sum l_s 2^(m_s - M), O = sum O_s 2^(m_s - M) / L,
+// lse = M + log2 L; rows no split found a key for give zeros (and lse 0).
+template <class Tr, int D>
+__global__ __launch_bounds__(D) void fa_fwd_combine_kernel(const FwdParams p, int tile_rows) {
+  const int prow = blockIdx.x % p.part_rows;
+  const int item = blockIdx.x / p.part_rows;
+  const int q_tile = item % p.num_q_tiles;
+  const int group = item / p.num_q_tiles;
+  const int row = q_tile * tile_rows + prow;
+  if (row >= p.q_len * p.group) return;
+  const int kv_head = group % p.num_kv_heads, b = group / p.num_kv_heads;
+  const int qi = row / p.group, head = kv_head * p.group + row % p.group;
+  const int d = threadIdx.x;
+  const int64_t slot0 = (int64_t)item * p.num_splits * p.part_rows + prow;
+  float m = -1e30f;
+  for (int s = 0; s < p.num_splits; s++) m = fmaxf(m, p.part_ml[(slot0 + (int64_t)s * p.part_rows) * 2]);
+  float l = 0.f, acc = 0.f;
+  for (int s = 0; s < p.num_splits; s++) {
+    const int64_t slot = slot0 + (int64_t)s * p.part_rows;
+    const float2 ml = *reinterpret_cast<const float2*>(p.part_ml + slot * 2);
+    const float w = ml.y > 0.f ? fast_exp2(ml.x - m) : 0.f;
+    l += ml.y * w;
+    acc += p.part_o[slot * D + d] * w;
+  }
+  const bool alive = l > 0.f;
+  const float value = alive ? acc / l : 0.f;
+  // 16-bit stores: pairs of neighbouring threads would need a shuffle to store 32 bits; the tensor
+  // is tiny in this mode
+  uint16_t* out = reinterpret_cast<uint16_t*>(p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh + (int64_t)qi * p.o_ss) * 2);
+  out[d] = (uint16_t)(Tr::pack2(value, 0.f) & 0xffff);
+  if (d == 0) p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qi] = alive ? m + fast_log2(l) : 0.f;
+}
+
+// How a forward call is run: in split mode (see fa_fwd_kernel) when the query sequence is shorter
+// than a work-group's 128 rows - the heads of a GQA group then fill the rows and share the key
+// tiles - or when one work-group per 128 query rows and head would occupy less than the chip's
+// 256 compute units.  The key sequence is divided so that about 1024 work-groups run, each with at
+// least four tiles.  Depends on the shapes only, so that the workspace can be sized up front.
+constexpr int kSplitTileRows = 128;  // (query, head) rows per work-group in split mode
+struct FwdPlan {
+  bool split_mode = false;
+  int num_splits = 1;
+  int part_rows = 0;
+  size_t part_o_bytes = 0, part_ml_bytes = 0;
+};
+FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv_heads, int head_dim) {
+  FwdPlan plan;
+  if (batch <= 0 || q_len <= 0 || kv_len <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return plan;
+  const int n_kv_tiles = cdiv(kv_len, kTileRows);
+  const int64_t regular = (int64_t)batch * num_heads * cdiv(q_len, kSplitTileRows);
+  const int ring_bytes = (2 * kTK * head_dim * 2 + 2 * kTK * 4) * (head_dim == 128 ? 2 : 3);
+  if (ring_bytes + live_tiles_bytes(4, n_kv_tiles) > 80 * 1024) return plan;
+  if (q_len >= kSplitTileRows && regular >= 256) return plan;
+  plan.split_mode = true;
+  const int64_t rows = (int64_t)q_len * (num_heads / num_kv_heads);
+  const int64_t items = (int64_t)batch * num_kv_heads * ((rows + kSplitTileRows - 1) / kSplitTileRows);
+  int splits = (int)((1024 + items - 1) / items);
+  splits = splits < n_kv_tiles / 4 ? splits : n_kv_tiles / 4;
+  splits = splits < 64 ? splits : 64;
+  plan.num_splits = splits > 1 ? splits : 1;
+  if (plan.num_splits > 1) {
+    plan.part_rows = (int)(rows < kSplitTileRows ? rows : kSplitTileRows);
+    const size_t slots = (size_t)items * plan.num_splits * plan.part_rows;
+    plan.part_o_bytes = (slots * head_dim * sizeof(float) + 15) / 16 * 16;
+    plan.part_ml_bytes = (slots * 2 * sizeof(float) + 15) / 16 * 16;
+  }
+  return plan;
+}
+
+template <class Tr, int D, int MQ, int NW, int WPS, int STAGES = 3, bool SPLIT = false>
 int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   FwdParams p = p0;
   constexpr int TQ = NW * 32 * MQ;
-  p.num_q_tiles = cdiv(p.q_len, TQ);
-  p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_q_tiles, p.group}.grid();
+  static_assert(!SPLIT || TQ == kSplitTileRows, "plan_forward() sizes the partial results for this tile");
+  if (SPLIT) {
+    p.num_q_tiles = cdiv(p.q_len * p.group, TQ);
+    p.total_items = p.batch * p.num_kv_heads * p.num_q_tiles * p.num_splits;
+  } else {
+    p.num_splits = 1;
+    p.num_q_tiles = cdiv(p.q_len, TQ);
+    p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_q_tiles, p.group}.grid();
+  }
   if (p.batch * p.num_heads * p.num_q_tiles == 0) return KVAX_OK;
-  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES>;
+  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES, SPLIT>;
   const int smem = FwdSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   constexpr int kWgPerCu = (WPS * 4 / NW) > 0 ? (WPS * 4 / NW) : 1;
   constexpr int kMaxSmem = 160 * 1024 / kWgPerCu;
@@ -372,7 +500,13 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
     configured = true;
   }
   hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
-  return check_launch("fa_fwd_kernel");
+  if (int rc = check_launch("fa_fwd_kernel")) return rc;
+  if (SPLIT && p.num_splits > 1) {
+    const int blocks = p.batch * p.num_kv_heads * p.num_q_tiles * p.part_rows;
+    hipLaunchKernelGGL((fa_fwd_combine_kernel<Tr, D>), dim3(blocks), dim3(D), 0, stream, p, TQ);
+    return check_launch("fa_fwd_combine_kernel");
+  }
+  return KVAX_OK;
 }
 
 // Two work-groups of four wavefronts per compute unit (each hides the other's prologue, barriers
@@ -381,6 +515,7 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
 template <class Tr, int D>
 int launch_fwd_auto(const FwdParams& p, hipStream_t stream) {
   constexpr int kStagesSmall = D == 128 ? 2 : 3;
+  if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall, true>(p, stream);
   const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
   if (small <= 80 * 1024) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
   return launch_fwd<Tr, D, 1, 8, 2, 3>(p, stream);
@@ -424,7 +559,9 @@ using namespace kvax;
 
 extern "C" size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* a) {
   if (!a || a->batch < 0 || a->kv_len < 0) return 0;
-  return tile_summary_bytes(a->batch, a->kv_len);  // kv tile summaries
+  // kv tile summaries, then the partial results of the split mode
+  const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim);
+  return tile_summary_bytes(a->batch, a->kv_len) + plan.part_o_bytes + plan.part_ml_bytes;
 }
 
 extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
@@ -466,6 +603,14 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.scale_log2 = fmaxf(fabsf(a->scale), 1e-30f) * 1.4426950408889634f;
   p.kv_tiles = (const int4*)workspace;
   p.n_kv_tiles = cdiv(a->kv_len, kTileRows);
+  {
+    const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim);
+    p.split_mode = plan.split_mode;
+    p.num_splits = plan.num_splits;
+    p.part_rows = plan.part_rows;
+    p.part_o = (float*)((char*)workspace + tile_summary_bytes(a->batch, a->kv_len));
+    p.part_ml = (float*)((char*)p.part_o + plan.part_o_bytes);
+  }
   hipStream_t stream = (hipStream_t)stream_;
   if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
   {

@@ -198,3 +198,32 @@ def test_errors(device):
             flash_attention(*data, ())
         with pytest.raises(ValueError):
             flash_attention(q[..., :48], k[..., :48], v[..., :48], q_pos, q_seg, kv_pos, kv_seg, mask)
+
+
+# Short query sequences run in the split mode: rows are (query, head) pairs of a GQA group and the
+# key sequence is divided over several work-groups whose partial results are merged.
+@pytest.mark.parametrize("sq, sk, hq, hkv, d, batch, pad, nseg", [
+    (1, 8192, 16, 4, 128, 2, 0, 1),       # decode, one row group per kv head
+    (1, 16384, 32, 8, 128, 4, 0, 1),      # decode at the benchmark's head layout
+    (1, 5000, 8, 8, 64, 3, 0, 1),         # decode, ragged key length, head_dim 64
+    (8, 4096, 32, 8, 128, 1, 0, 1),       # a few new tokens (32 rows per kv head)
+    (48, 2048, 16, 4, 128, 2, 0, 1),      # 192 rows per kv head: two row tiles
+    (200, 3000, 6, 2, 64, 1, 37, 3),      # ragged prefill chunk with documents and padding
+    (128, 1024, 4, 1, 128, 1, 100, 2),    # multi-query attention
+])
+def test_split_mode_matches_dense_oracle(device, sq, sk, hq, hkv, d, batch, pad, nseg):
+    lengths = generate_random_segments_lengths(sk, nseg)
+    start = sk - sq - pad
+    data, scale = make_random_attention_inputs(batch, sq, sk, hq, hkv, d, d, seed=sq + sk,
+                                               num_pad_tokens=pad, start_query_position=start,
+                                               device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    if lengths is not None:  # documents over the keys; each query takes the document of its position
+        bounds = np.cumsum([0] + lengths)
+        seg_of = np.searchsorted(bounds, np.arange(sk), side="right") - 1
+        kv_seg = torch.where(kv_seg == -1, kv_seg, torch.from_numpy(seg_of).to(torch.int32).to(device)[None])
+        q_seg = torch.where(q_seg == -1, q_seg,
+                            torch.from_numpy(seg_of).to(torch.int32).to(device)[q_pos.clamp(max=sk - 1).long()])
+        data = (q, k, v, q_pos, q_seg, kv_pos, kv_seg)
+    out = run_forward(data, scale, 128, 128)
+    check(out, oracle_forward(data, scale), data[4])
