@@ -22,6 +22,7 @@ import numpy as np
 import torch
 
 MFMA_BF16_DENSE_PEAK_TFLOPS = 2516.6  # MI355X datasheet: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+HBM_PEAK_GBPS = 8000.0                # MI355X datasheet: HBM3E
 CALIBRATION_BYTES = 1 << 30            # bytes read (and bytes written) by the --pmc-calibration kernel
 ROOT = os.path.dirname(os.path.abspath(__file__))
 
@@ -49,6 +50,8 @@ WORKLOAD_TEXT = {
                 "document mask (lognormal median 4096), forward+backward, one CP=8 shard",
     "block_skip": "block_skip: B4 S16384 Hq64/Hkv8 D128 bf16, bidirectional document mask, exponential "
                   "document lengths (mean 512, min 32), 20-30% padding per row, forward+backward",
+    "decode32k": "decode32k: B8, one query per row against a 32768-slot key cache filled to 16384..32764 "
+                 "keys (the rest padding), Hq32/Hkv8 D128 bf16, forward only (split mode)",
 }
 
 
@@ -125,6 +128,7 @@ def main():
                  block=args.block)
     tensors = w.draw_tensors(args.seed, dev, with_dout=True)
     q, k, v, dout = tensors
+    decode = w.q_len == 1
     ids = w.ids(dev)
     fp, bp = FlashAttentionParamsConfig(*w.fwd_blocks), FlashAttentionParamsConfig(*w.bwd_blocks)
     specs = (("data", None, "model", None), ("data", None, "model", None))
@@ -207,6 +211,21 @@ def main():
     kernel_flops = {"fa_fwd_kernel": f_fwd, "fa_bwd_dq_kernel": 1.5 * f_fwd, "fa_bwd_dkdv_kernel": 2.0 * f_fwd}
     dominant = max(kernel_ms, key=kernel_ms.get)
     achieved = kernel_flops[dominant] / (kernel_ms[dominant] * 1e-3) / 1e12
+    if decode:
+        # one query per row: the kernel has to read every attendable key and value once (all query
+        # heads of a group share them) plus Q, and write O and lse; HBM is the roof
+        alg_bytes = (2 * pairs * w.num_kv_heads * w.head_dim * 2
+                     + 2 * w.batch * w.num_heads * w.head_dim * 2 + w.batch * w.num_heads * 4)
+        gbps = alg_bytes / (kernel_ms["fa_fwd_kernel"] * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "kernel": "fa_fwd_kernel (split mode) + fa_fwd_combine_kernel",
+                    "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                    "traffic": recorded_traffic("fa_fwd_kernel", args.workload),
+                    "algorithmic_bytes": alg_bytes}
+    else:
+        roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved,
+                    "peak": MFMA_BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
+                    "traffic": recorded_traffic(dominant, args.workload)}
     result = {
         "metric": "doc-mask attention TFLOP/s, forward+backward, 32k tokens, bf16, unmasked FLOPs"
                   if backward else "doc-mask attention TFLOP/s, forward, bf16, unmasked FLOPs",
@@ -231,15 +250,7 @@ def main():
             "num_documents": len(w.meta.get("doc_lengths", [])) or None,
             "padding_tokens": w.meta.get("pad"),
         },
-        "roofline": {
-            "bound": "mfma",
-            "kernel": dominant,
-            "achieved": achieved,
-            "peak": MFMA_BF16_DENSE_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
-            "traffic": recorded_traffic(dominant, args.workload),
-        },
+        "roofline": roofline,
         "step_frac_of_mfma_peak": value / MFMA_BF16_DENSE_PEAK_TFLOPS,
         "fwd_tflops": f_fwd / (kernel_ms["fa_fwd_kernel"] * 1e-3) / 1e12,
         "mask_build_ms": mask_ms,

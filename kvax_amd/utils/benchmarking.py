@@ -239,6 +239,8 @@ def workload(name: str, seed: int = 0, restart_positions: bool = True, cp_rank: 
                        all 131072 tokens; lognormal documents (median 4096), forward + backward
     ``block_skip``     B4 S16384 64/8 D128 bf16, exponential documents (mean 512, min 32), 20-30 %
                        padding per row, bidirectional (constant positions), forward + backward
+    ``decode32k``      B8, one query per row against a 32768-slot key cache, 32/8 D128 bf16; row i has
+                       16384 + i * 2340 keys filled, the rest of the cache is padding; forward only
     """
     rng = np.random.default_rng(seed)
     if name == "cpu_plumbing":
@@ -292,6 +294,15 @@ def workload(name: str, seed: int = 0, restart_positions: bool = True, cp_rank: 
         pos, seg = np.stack(pos_rows), np.stack(seg_rows)
         return Workload(name, B, S, S, 64, 8, 128, False, (block, block), (block, block), True,
                         pos, seg, pos.copy(), seg.copy(), meta=dict(seed=seed, rows=metas))
+    if name == "decode32k":
+        B, S = 8, 32768
+        filled = np.array([16384 + i * 2340 for i in range(B)], np.int32)  # 16384 ... 32764
+        kv_pos = np.broadcast_to(np.arange(S, dtype=np.int32), (B, S)).copy()
+        kv_seg = np.where(kv_pos < filled[:, None], 0, PADDING_SEGMENT_ID).astype(np.int32)
+        q_pos = (filled - 1)[:, None].astype(np.int32)
+        q_seg = np.zeros((B, 1), np.int32)
+        return Workload(name, B, 1, S, 32, 8, 128, True, (block, block), (block, block), False,
+                        q_pos, q_seg, kv_pos, kv_seg, meta=dict(seed=seed, filled=filled.tolist()))
     raise ValueError(f"unknown workload {name!r}")
 
 

@@ -227,3 +227,13 @@ def test_split_mode_matches_dense_oracle(device, sq, sk, hq, hkv, d, batch, pad,
         data = (q, k, v, q_pos, q_seg, kv_pos, kv_seg)
     out = run_forward(data, scale, 128, 128)
     check(out, oracle_forward(data, scale), data[4])
+
+
+def test_decode_workload_all_rows(device):
+    """The decode measurement workload (one query per row, key caches filled to different lengths)
+    against the oracle, every batch row and head."""
+    w = workload("decode32k")
+    q, k, v = w.draw_tensors(0, device, with_dout=False)
+    data = (q, k, v, *w.ids(device))
+    out = run_forward(data, w.scale, *w.fwd_blocks)
+    check(out, oracle_forward(data, w.scale), data[4])
