@@ -135,7 +135,9 @@ typedef struct kvax_fa_args {
 
 /* Workspaces (16-byte aligned device memory, contents undefined on entry, reusable right after the
  * call's work on `stream`):
- *   forward:  32 bytes per 64-row kv tile and batch row (tile summaries used to skip dead tiles);
+ *   forward:  32 bytes per 64-row kv tile and batch row (tile summaries used to skip dead tiles),
+ *             plus, for short query sequences, the fp32 partial results of the work-groups that
+ *             share one key sequence (a function of the shapes only);
  *   backward: delta [batch, num_heads, q_len] fp32, the tile summaries of the kv and the query
  *             sequence, and the dispatch order of the dK/dV work items (longest first). */
 size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* args);
