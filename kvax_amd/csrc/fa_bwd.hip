@@ -430,7 +430,10 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
                             live_bits + wave * words, word0, lane);
   __syncthreads();
   if (wave == 0)
-    compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
+    // highest query tile first: every kv work-group of a document ends on the document's last query
+    // tiles, so walking backwards the work-groups that run together stream the same Q/dO tiles at
+    // the same time (they start at different tiles when walking forwards) and share them in L2
+    compact_live_tiles<NW, true>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
   __syncthreads();
   const int n_live = *live_count;
   const int steps = n_live * p.group;  // every head of the group walks the same list

@@ -193,14 +193,16 @@ __device__ __forceinline__ void mark_live_tiles(const int4* tiles, const TilePar
 }
 
 // Compacts the NW per-wave bitmaps into a list of the tiles that are live for at least one
-// wavefront: entry = tile index | (mask of the waves it is live for) << 24.  Executed by one
-// wavefront; the number of entries is written to *count.
-template <int NW>
+// wavefront: entry = tile index | (mask of the waves it is live for) << 24, in ascending tile order
+// (DESCENDING: highest tile first).  Executed by one wavefront; the number of entries is written
+// to *count.
+template <int NW, bool DESCENDING = false>
 __device__ __forceinline__ void compact_live_tiles(const unsigned long long* bits, int words, int word0,
                                                    uint32_t* list, int* count, int lane) {
   static_assert(NW <= 8, "the wave mask is stored in the top byte of an entry");
   int n = 0;
-  for (int w = 0; w < words; w++) {
+  for (int k = 0; k < words; k++) {
+    const int w = DESCENDING ? words - 1 - k : k;
     unsigned long long any = 0;
     uint32_t waves = 0;
 #pragma unroll
@@ -209,8 +211,10 @@ __device__ __forceinline__ void compact_live_tiles(const unsigned long long* bit
       any |= m;
       waves |= (uint32_t)((m >> lane) & 1) << i;
     }
+    // entries of this word before the lane's own: set bits below it (ascending) or above it
+    const unsigned long long before = DESCENDING ? (any >> lane) >> 1 : any & ((1ull << lane) - 1);
     if ((any >> lane) & 1)
-      list[n + __popcll(any & ((1ull << lane) - 1))] = (uint32_t)((word0 + w) * 64 + lane) | (waves << 24);
+      list[n + __popcll(before)] = (uint32_t)((word0 + w) * 64 + lane) | (waves << 24);
     n += __popcll(any);
   }
   if (lane == 0) *count = n;
