@@ -194,3 +194,64 @@ def test_key_sequence_too_long_for_two_work_groups_per_cu(device):
     for name, got, ref in (("dq", dq, ref_dq), ("dk", dk, ref_dk), ("dv", dv, ref_dv)):
         assert np.abs(f(got) - ref).max() <= 2e-2, name
     assert (f(dk)[0, :70000] == 0).all() and (f(dv)[0, :70000] == 0).all()
+
+
+def test_hip_graph_replays_match_eager(device):
+    """Forward + backward recorded once into a HIP graph and replayed on new inputs: the entry
+    points enqueue kernels only (no allocation, no synchronisation, no memset), so every replay
+    must equal the eager result on the same inputs - with eager work and synchronisations between
+    the replays."""
+    data, scale = make_random_attention_inputs(2, 2304, 2304, 8, 2, 128, 128, seed=9, num_pad_tokens=200,
+                                               list_of_segment_lengths=[700, 900, -1], device=device)
+    q, k, v, *ids = data
+    p = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(*ids, fwd_params=p, bwd_params=p, calc_bwd_mask=True)
+    dout = torch.randn_like(q)
+
+    def eager(q_, k_, v_, do_):
+        out, lse = flash_attention_forward(q_, k_, v_, *ids, masks[0], scale, p, p)
+        return (out, *flash_attention_backward(q_, k_, v_, *ids, masks[1], masks[2], out, lse, do_, scale, p, p))
+
+    eager(q, k, v, dout)  # first call configures the kernels' LDS limits, which cannot be captured
+    sq, sk, sv, sdo = (t.clone() for t in (q, k, v, dout))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        results = eager(sq, sk, sv, sdo)
+    for seed in (1, 2, 3):
+        g = torch.Generator().manual_seed(seed)
+        new = [torch.randn(t.shape, generator=g).to(t.dtype).to(device) for t in (q, k, v, dout)]
+        for static, fresh in zip((sq, sk, sv, sdo), new):
+            static.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = eager(*new)
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("out", "dq", "dk", "dv"), results, want):
+            assert torch.equal(got, ref), f"{name}, replay {seed}"
+
+
+def test_hip_graph_replays_of_the_split_forward(device):
+    """Same for a decoding step (split mode: partial results in the workspace, combine kernel)."""
+    data, scale = make_random_attention_inputs(4, 1, 4096, 16, 4, 128, 128, seed=5,
+                                               start_query_position=(4000, 100, 2047, 3000), device=device)
+    q, k, v, *ids = data
+    p = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(*ids, fwd_params=p)
+    eager = lambda q_, k_, v_: flash_attention_forward(q_, k_, v_, *ids, masks[0], scale, p, p)[0]
+    eager(q, k, v)
+    sq, sk, sv = (t.clone() for t in (q, k, v))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        result = eager(sq, sk, sv)
+    for seed in (1, 2, 3):
+        g = torch.Generator().manual_seed(seed)
+        new = [torch.randn(t.shape, generator=g).to(t.dtype).to(device) for t in (q, k, v)]
+        for static, fresh in zip((sq, sk, sv), new):
+            static.copy_(fresh)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(result, eager(*new)), f"replay {seed}"
