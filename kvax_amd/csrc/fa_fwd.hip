@@ -52,8 +52,10 @@ struct FwdParams {
   uint32_t q_sign;       // 0x80008000 when the scale is negative: Q is negated on load
   float scale_log2;      // |scale| * log2(e), > 0
   // split mode (short query sequences, see fa_fwd_kernel): rows are (query, head of the group)
-  // pairs; each work-group takes 1 / num_splits of the live kv tiles and leaves a partial result
-  int num_splits, part_rows;  // rows per tile that have a partial (<= TQ)
+  // pairs; work-group `split` of an item takes the kv tiles [split, split + 1) * split_tiles of the
+  // item's range and leaves a partial result
+  int num_splits, split_tiles;
+  int part_rows;              // rows per tile that have a partial (<= TQ)
   float* part_o;              // [items, num_splits, part_rows, D] unnormalised O
   float* part_ml;             // [items, num_splits, part_rows, 2] running max (base 2) and sum
 };
@@ -72,8 +74,10 @@ struct FwdSmem {
 // SPLIT (short query sequences, e.g. decoding one token against a long key sequence, where one
 // work-group per (batch, head) would leave most of the chip idle and read the keys serially): the
 // rows of a work-group are (query, query head) pairs of one (batch, kv head) - all heads of a GQA
-// group share the key tiles they stream - and the live kv tiles are divided over num_splits
-// work-groups, each leaving an unnormalised partial result that fa_fwd_combine_kernel merges.
+// group share the key tiles they stream - and the kv range of the block mask is cut into windows of
+// split_tiles tiles, one work-group each (those beyond the end of the range have nothing to do), each
+// leaving an unnormalised partial result that fa_fwd_combine_kernel merges.  Windows of one size
+// for all rows of the batch keep the work-groups equally long when the rows are not.
 template <class Tr, int D, int MQ, int NW, int WPS, int STAGES, bool SPLIT>
 __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p) {
   using vec8 = typename Tr::vec8;
@@ -137,8 +141,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     }
   }
   hi = min(hi, p.kv_len);
-  const int t_lo = lo / kTK;
-  const int t_hi = hi > lo ? (hi + kTK - 1) / kTK : t_lo;
+  int t_lo = lo / kTK;
+  int t_hi = hi > lo ? (hi + kTK - 1) / kTK : t_lo;
+  if (SPLIT) {  // this work-group's window of the range
+    t_lo = min(t_lo + split * p.split_tiles, t_hi);
+    t_hi = min(t_lo + p.split_tiles, t_hi);
+  }
   const int tf_lo = (flo + kTK - 1) / kTK, tf_hi = fhi / kTK;
 
   // ---- per-lane query columns ------------------------------------------------------------
@@ -182,9 +190,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
   __syncthreads();
   const int n_live = *live_count;
-  // this work-group's share of the live tiles
-  const int i_lo = SPLIT ? (int)((int64_t)n_live * split / p.num_splits) : 0;
-  const int i_hi = SPLIT ? (int)((int64_t)n_live * (split + 1) / p.num_splits) : n_live;
+  const int i_lo = 0, i_hi = n_live;
 
   f32x16 o[DT][MQ];
   float m_run[MQ], l_run[MQ];
@@ -440,15 +446,14 @@ __global__ __launch_bounds__(D) void fa_fwd_combine_kernel(const FwdParams p, in
 // How a forward call is run: in split mode (see fa_fwd_kernel) when the query sequence is shorter
 // than a work-group's 128 rows - the heads of a GQA group then fill the rows and share the key
 // tiles - or when one work-group per 128 query rows and head would occupy less than the chip's
-// 256 compute units.  The key sequence is divided so that about 1024 work-groups run (two rounds
-// of two per compute unit: with 512 a batch of equally long rows is 4 % faster, one of unequal rows
-// 5-8 % slower, because every row is cut into the same number of parts), each with at least four
-// tiles.  Depends on the shapes only, so that the workspace can be sized up front.
+// 256 compute units.  The key sequence is cut into windows of at least four tiles, about 1024 over
+// the whole batch (two rounds of two work-groups per compute unit).  Depends on the shapes only, so
+// that the workspace can be sized up front.
 constexpr int kSplitTileRows = 128;  // (query, head) rows per work-group in split mode
 constexpr int kSplitWorkGroups = 1024;
 struct FwdPlan {
   bool split_mode = false;
-  int num_splits = 1;
+  int num_splits = 1, split_tiles = 0;
   int part_rows = 0;
   size_t part_o_bytes = 0, part_ml_bytes = 0;
 };
@@ -463,10 +468,12 @@ FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv
   plan.split_mode = true;
   const int64_t rows = (int64_t)q_len * (num_heads / num_kv_heads);
   const int64_t items = (int64_t)batch * num_kv_heads * ((rows + kSplitTileRows - 1) / kSplitTileRows);
-  int splits = (int)((kSplitWorkGroups + items - 1) / items);
-  splits = splits < n_kv_tiles / 4 ? splits : n_kv_tiles / 4;
-  splits = splits < 64 ? splits : 64;
-  plan.num_splits = splits > 1 ? splits : 1;
+  // windows of one size for every item: about kSplitWorkGroups of them if every range were full
+  int window = (int)((items * n_kv_tiles + kSplitWorkGroups - 1) / kSplitWorkGroups);
+  window = window > 4 ? window : 4;
+  window = window > cdiv(n_kv_tiles, 64) ? window : cdiv(n_kv_tiles, 64);
+  plan.split_tiles = window;
+  plan.num_splits = cdiv(n_kv_tiles, window);
   if (plan.num_splits > 1) {
     plan.part_rows = (int)(rows < kSplitTileRows ? rows : kSplitTileRows);
     const size_t slots = (size_t)items * plan.num_splits * plan.part_rows;
@@ -612,6 +619,7 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
     const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim);
     p.split_mode = plan.split_mode;
     p.num_splits = plan.num_splits;
+    p.split_tiles = plan.split_tiles;
     p.part_rows = plan.part_rows;
     p.part_o = (float*)((char*)workspace + tile_summary_bytes(a->batch, a->kv_len));
     p.part_ml = (float*)((char*)p.part_o + plan.part_o_bytes);
