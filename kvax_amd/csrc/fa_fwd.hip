@@ -13,10 +13,12 @@
 // B-operand layout of the second contraction O^T += V^T P^T -- P never goes through LDS.  V^T
 // operands are gathered from the row-major V tile with transposing LDS reads.  K/V tiles reach
 // LDS by asynchronous global->LDS copies (no registers involved) into a ring of swizzled stages,
-// two tiles ahead of the one being consumed, and are shared by the work-group's 8 wavefronts
-// (256 query rows); the query heads of one GQA group run as neighbouring work-groups on one XCD
-// so K/V tiles are served from that XCD's L2.  Tiles of the block-mask range in which no
-// (query, key) pair can pass the element mask are dropped up front (fa_tiles.hip).
+// one or two tiles ahead of the one being consumed, and are shared by the work-group's 4 or 8
+// wavefronts (128 or 256 query rows); the query heads of one GQA group run as neighbouring
+// work-groups on one XCD so K/V tiles are served from that XCD's L2.  Tiles of the block-mask range
+// in which no (query, key) pair can pass the element mask are dropped up front (fa_tiles.hip).
+// Short query sequences (decoding) run in a split mode that divides the key sequence over
+// work-groups and merges their partial results (see fa_fwd_kernel).
 #include "common.h"
 #include "fa_common.h"
 
