@@ -369,6 +369,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   // ---- split mode with several splits: leave the unnormalised partial result ---------------
   if (SPLIT && p.num_splits > 1) {
     const int prow = wave * 32 + c;  // MQ == 1
+    const float l_row = l_run[0] + xor32(l_run[0]);  // cross-lane: outside the divergent branch
     if (row_in[0] && prow < p.part_rows) {
       const int64_t slot = ((int64_t)item * p.num_splits + split) * p.part_rows + prow;
       float* po = p.part_o + slot * D;
@@ -378,8 +379,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
         for (int g4 = 0; g4 < 4; g4++)
           *reinterpret_cast<float4*>(po + 32 * dt + 8 * g4 + 4 * h) =
               make_float4(o[dt][0][4 * g4 + 0], o[dt][0][4 * g4 + 1], o[dt][0][4 * g4 + 2], o[dt][0][4 * g4 + 3]);
-      const float l = l_run[0] + xor32(l_run[0]);
-      if (h == 0) *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], l);
+      if (h == 0) *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], l_row);
     }
     return;
   }

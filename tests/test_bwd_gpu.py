@@ -201,3 +201,60 @@ def test_missing_backward_masks(device):
         out = flash_attention(q, k, v, *ids, mask, scale=scale)
         with pytest.raises(ValueError):
             out.sum().backward()
+
+
+def _random_case(seed):
+    """Seeded random shapes, documents, padding, block sizes and head layouts."""
+    rng = np.random.default_rng(seed)
+    d = int(rng.choice([64, 128]))
+    hkv = int(rng.choice([1, 2, 4]))
+    hq = hkv * int(rng.choice([1, 2, 4, 8]))
+    block = int(rng.choice([64, 128]))
+    sq = block * int(rng.integers(1, 2048 // block + 1))
+    sk = sq if rng.random() < 0.6 else block * int(rng.integers(1, 3072 // block + 1))
+    batch = int(rng.integers(1, 4))
+    n = min(sq, sk)
+    nseg = int(rng.integers(1, 7))
+    cuts = np.sort(rng.choice(np.arange(1, n), size=min(nseg - 1, n - 1), replace=False)) if nseg > 1 else []
+    lengths = np.diff(np.concatenate([[0], cuts, [n]])).astype(int).tolist()
+    pad = int(rng.integers(0, n // 2)) if rng.random() < 0.5 else 0
+    return dict(batch=batch, sq=sq, sk=sk, hq=hq, hkv=hkv, d=d, block=block, lengths=lengths, pad=pad,
+                restart=bool(rng.random() < 0.5))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_randomized_shapes_forward_and_backward(device, seed):
+    c = _random_case(seed)
+    data, scale = make_random_attention_inputs(c["batch"], c["sq"], c["sk"], c["hq"], c["hkv"], c["d"], c["d"],
+                                               seed=seed, num_pad_tokens=c["pad"],
+                                               list_of_segment_lengths=c["lengths"], device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    # tokens beyond the laid-out documents form one more document: segment ids must not come back to
+    # an earlier value along a sequence (the block-mask heuristic of the reference assumes that)
+    n, last = min(c["sq"], c["sk"]), len(c["lengths"])
+    q_seg, kv_seg = q_seg.clone(), kv_seg.clone()
+    q_seg[:, n:] = torch.where(q_seg[:, n:] == -1, -1, last)
+    kv_seg[:, n:] = torch.where(kv_seg[:, n:] == -1, -1, last)
+    data = (q, k, v, q_pos, q_seg, kv_pos, kv_seg)
+    if c["restart"]:  # positions restart in every document (the regime in which the masks over-cover)
+        def restart(pos, seg):
+            out = pos.clone()
+            for b in range(seg.shape[0]):
+                s = seg[b].cpu().numpy()
+                starts = np.r_[0, np.nonzero(np.diff(s))[0] + 1]
+                first = np.zeros(len(s), np.int64)
+                first[starts] = starts
+                first = np.maximum.accumulate(first)
+                out[b] = torch.from_numpy(np.arange(len(s)) - first).to(pos.dtype)
+            return out
+        q_pos, kv_pos = restart(q_pos, q_seg), restart(kv_pos, kv_seg)
+        data = (q, k, v, q_pos, q_seg, kv_pos, kv_seg)
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(seed)).to(torch.bfloat16).to(device)
+    blocks = (c["block"], c["block"])
+    out, dq, dk, dv = run_backward(data, scale, blocks, blocks, dout)
+    q_, k_, v_, *ids_ = [x.cpu() for x in data]
+    ref_out, _ = ao.attention_forward(q_.float().numpy(), k_.float().numpy(), v_.float().numpy(),
+                                      *[x.numpy() for x in ids_], scale)
+    assert np.abs(out.float().cpu().numpy() - ref_out).max() <= ATOL, c
+    refs = oracle_backward(data, scale, dout)
+    check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if c["hq"] // c["hkv"] >= 8 else ATOL)
