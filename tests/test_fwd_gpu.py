@@ -237,3 +237,47 @@ def test_decode_workload_all_rows(device):
     data = (q, k, v, *w.ids(device))
     out = run_forward(data, w.scale, *w.fwd_blocks)
     check(out, oracle_forward(data, w.scale), data[4])
+
+
+def _short_query_case(seed):
+    """Seeded random decoding / chunked-prefill inputs: the queries are the last tokens of a key
+    cache filled to a random length (the rest is padding), documents with monotone ids over the
+    cache, positions global or restarting per document, some trailing query padding."""
+    rng = np.random.default_rng(1000 + seed)
+    d = int(rng.choice([64, 128]))
+    hkv = int(rng.choice([1, 2, 8]))
+    hq = hkv * int(rng.choice([1, 2, 4, 8, 16]))
+    batch = int(rng.integers(1, 5))
+    sq = int(rng.choice([1, 1, 2, 5, 8, 17, 64, 100, 200]))
+    sk = int(rng.integers(max(sq, 65), 7000))
+    block = int(rng.choice([64, 128]))
+    restart = bool(rng.random() < 0.5)
+    kv_seg = np.zeros((batch, sk), np.int32); kv_pos = np.zeros((batch, sk), np.int32)
+    q_seg = np.zeros((batch, sq), np.int32); q_pos = np.zeros((batch, sq), np.int32)
+    for b in range(batch):
+        filled = int(rng.integers(sq, sk + 1))
+        ndoc = int(rng.integers(1, 6))
+        cuts = (np.sort(rng.choice(np.arange(1, filled), size=min(ndoc - 1, filled - 1), replace=False))
+                if ndoc > 1 and filled > 1 else np.array([], int))
+        seg = np.searchsorted(cuts, np.arange(filled), side="right").astype(np.int32)
+        pos = np.arange(filled, dtype=np.int32)
+        if restart:
+            pos = pos - np.r_[0, cuts][seg].astype(np.int32)
+        kv_seg[b, :filled], kv_seg[b, filled:] = seg, -1
+        kv_pos[b, :filled], kv_pos[b, filled:] = pos, np.arange(sk - filled)
+        q_seg[b], q_pos[b] = seg[filled - sq:], pos[filled - sq:]
+        if rng.random() < 0.3 and sq > 2:
+            q_seg[b, sq - int(rng.integers(1, sq)):] = -1
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(batch, sq, hq, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(batch, sk, hkv, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(batch, sk, hkv, d, generator=g).to(torch.bfloat16)
+    ids = tuple(torch.from_numpy(x) for x in (q_pos, q_seg, kv_pos, kv_seg))
+    return (q, k, v, *ids), d ** -0.5, block
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_randomized_short_query_shapes(device, seed):
+    data, scale, block = _short_query_case(seed)
+    out = run_forward(tuple(x.to(device) for x in data), scale, block, block)
+    check(out, oracle_forward(data, scale), data[4])
