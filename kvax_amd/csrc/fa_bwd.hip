@@ -722,7 +722,7 @@ template <class Tr, int D, int NW, int STAGES>
 int launch_dq(BwdParams p, hipStream_t stream) {
   auto kernel = fa_bwd_dq_kernel<Tr, D, NW, 2, STAGES>;
   static bool done = false;
-  constexpr int kLimit = 160 * 1024 / (8 / NW);
+  constexpr int kLimit = kLdsPerCu / (8 / NW);
   const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   if (int rc = reserve_lds(kernel, smem, kLimit, &done, "the dQ kernel")) return rc;
   p.num_tiles = cdiv(p.q_len, NW * 32);
@@ -746,7 +746,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   const bool run_dq = p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ);
   const bool run_dkdv = p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV);
   const bool dq_small =
-      DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles) <= 80 * 1024;
+      DqSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles) <= kLdsHalfCu;
   // dK/dV runs one long work-group per compute unit: its light work items are dispatched last, by
   // decreasing number of live tiles, so that the launch does not end on a few long ones
   {
@@ -772,7 +772,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2>;
     static bool done = false;
     // live-tile bookkeeping for as many query tiles as the remaining LDS holds (a multiple of 64)
-    constexpr int kLdsLimit = 160 * 1024;
+    constexpr int kLdsLimit = kLdsPerCu;
     int chunk = 64;
     while (chunk < p.n_q_tiles && DkdvSmem<D>::kTotal + live_tiles_bytes(NW, chunk * 2) <= kLdsLimit) chunk *= 2;
     p.list_tiles = min(chunk, max(p.n_q_tiles, 1));

@@ -220,6 +220,10 @@ __device__ __forceinline__ void compact_live_tiles(const unsigned long long* bit
   if (lane == 0) *count = n;
 }
 
+// LDS of a gfx950 compute unit, and the share of each work-group when two run per compute unit.
+constexpr int kLdsPerCu = 160 * 1024;
+constexpr int kLdsHalfCu = kLdsPerCu / 2;
+
 // LDS bytes for the live-tile bookkeeping of a range of at most `tiles` tiles.
 __host__ __device__ constexpr int live_tiles_bytes(int nw, int tiles) {
   return 16 + nw * ((tiles + 63) / 64 + 1) * 8 + tiles * 4;

@@ -465,7 +465,7 @@ FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv
   const int n_kv_tiles = cdiv(kv_len, kTileRows);
   const int64_t regular = (int64_t)batch * num_heads * cdiv(q_len, kSplitTileRows);
   const int ring_bytes = (2 * kTK * head_dim * 2 + 2 * kTK * 4) * (head_dim == 128 ? 2 : 3);
-  if (ring_bytes + live_tiles_bytes(4, n_kv_tiles) > 80 * 1024) return plan;
+  if (ring_bytes + live_tiles_bytes(4, n_kv_tiles) > kLdsHalfCu) return plan;
   if (q_len >= kSplitTileRows && regular >= 256) return plan;
   plan.split_mode = true;
   const int64_t rows = (int64_t)q_len * (num_heads / num_kv_heads);
@@ -502,7 +502,7 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES, SPLIT>;
   const int smem = FwdSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   constexpr int kWgPerCu = (WPS * 4 / NW) > 0 ? (WPS * 4 / NW) : 1;
-  constexpr int kMaxSmem = 160 * 1024 / kWgPerCu;
+  constexpr int kMaxSmem = kLdsPerCu / kWgPerCu;
   if (smem > kMaxSmem)
     return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
                 p.kv_len, smem, kMaxSmem);
@@ -531,7 +531,7 @@ int launch_fwd_auto(const FwdParams& p, hipStream_t stream) {
   constexpr int kStagesSmall = D == 128 ? 2 : 3;
   if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall, true>(p, stream);
   const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
-  if (small <= 80 * 1024) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
+  if (small <= kLdsHalfCu) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
   return launch_fwd<Tr, D, 1, 8, 2, 3>(p, stream);
 }
 
