@@ -177,3 +177,35 @@ def test_mask_picture_of_a_sharded_mask():
     assert levels.tolist() == [[1, 1, 1, 0], [0, 1, 1, 1]]
     with pytest.raises(ValueError):
         mask_block_levels(AttentionMask(lower, upper, zeros, zeros), 3)
+
+
+def _fa_args(batch, q_len, kv_len, heads, kv_heads, head_dim):
+    a = _native.FaArgs()
+    a.batch, a.q_len, a.kv_len = batch, q_len, kv_len
+    a.num_heads, a.num_kv_heads, a.head_dim = heads, kv_heads, head_dim
+    return a
+
+
+def test_workspace_sizes_follow_the_shapes():
+    """The workspace functions are pure functions of the shapes (no GPU needed): 32 bytes per
+    64-row tile and batch row for the summaries; the forward adds room for partial results only
+    where it runs in its split mode (short query sequences); the backward holds delta, both
+    summaries and the dispatch order of the dK/dV work items."""
+    lib = _native.lib()
+    fwd = lambda *s: lib.kvax_fa_fwd_workspace_bytes(ctypes.byref(_fa_args(*s)))
+    bwd = lambda *s: lib.kvax_fa_bwd_workspace_bytes(ctypes.byref(_fa_args(*s)))
+    assert fwd(1, 32768, 32768, 32, 8, 128) == 32 * 512                 # training shape: summaries only
+    assert fwd(4, 8192, 8192, 16, 16, 128) == 4 * 32 * 128
+    summaries = 8 * 32 * 512
+    decode = fwd(8, 1, 32768, 32, 8, 128)                               # one query per row: split mode
+    assert decode > summaries
+    partial_bytes = decode - summaries
+    # 64 work items (8 rows x 8 kv heads) x windows x 4 rows x (128 + 2) floats, 16-byte aligned pieces
+    assert partial_bytes % (64 * 4 * 4) == 0
+    windows = partial_bytes // (64 * 4 * (128 + 2) * 4)
+    assert 2 <= windows <= 64 and windows * 64 * 4 * 130 * 4 == partial_bytes
+    assert fwd(8, 1, 64, 32, 8, 128) == 8 * 32                          # too short to divide
+    assert fwd(0, 1, 32768, 32, 8, 128) == 0
+    delta = 1 * 32 * 32768 * 4
+    order = (2 * 256 + 1) * 4 + 12                                      # 256 kv work items, padded to 16
+    assert bwd(1, 32768, 32768, 32, 8, 128) == delta + 2 * 32 * 512 + order
