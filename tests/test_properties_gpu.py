@@ -255,3 +255,34 @@ def test_hip_graph_replays_of_the_split_forward(device):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(result, eager(*new)), f"replay {seed}"
+
+
+def test_strided_views_give_the_same_bits_as_contiguous_tensors(device):
+    """Q, K, V taken as views of one fused projection output ([B, S, (Hq + 2 Hkv) * D]) and dO as a
+    transposed [B, H, S, D] tensor: the kernels read through strides, so outputs and gradients equal
+    those for contiguous copies bit for bit (and no hidden copy is needed)."""
+    b, s, hq, hkv, d = 2, 1024, 8, 2, 128
+    g = torch.Generator().manual_seed(31)
+    fused = torch.randn(b, s, (hq + 2 * hkv) * d, generator=g).to(torch.bfloat16).to(device)
+    q = fused[..., :hq * d].view(b, s, hq, d)
+    k = fused[..., hq * d:(hq + hkv) * d].view(b, s, hkv, d)
+    v = fused[..., (hq + hkv) * d:].view(b, s, hkv, d)
+    dout = torch.randn(b, hq, s, d, generator=g).to(torch.bfloat16).to(device).transpose(1, 2)
+    assert not q.is_contiguous() and not k.is_contiguous() and not dout.is_contiguous()
+    _, _, _, q_pos, q_seg, kv_pos, kv_seg = make_random_attention_inputs(
+        b, s, s, hq, hkv, d, d, seed=1, num_pad_tokens=90, list_of_segment_lengths=[300, 500, -1],
+        device=device)[0]
+    ids = (q_pos, q_seg, kv_pos, kv_seg)
+    p = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(*ids, fwd_params=p, bwd_params=p, calc_bwd_mask=True)
+    scale = d ** -0.5
+
+    def run(q_, k_, v_, do_):
+        out, lse = flash_attention_forward(q_, k_, v_, *ids, masks[0], scale, p, p)
+        return (out, *flash_attention_backward(q_, k_, v_, *ids, masks[1], masks[2], out, lse, do_, scale, p, p))
+
+    strided = run(q, k, v, dout)
+    dense = run(q.contiguous(), k.contiguous(), v.contiguous(), dout.contiguous())
+    for name, a, c in zip(("out", "dq", "dk", "dv"), strided, dense):
+        assert torch.equal(a, c), name
