@@ -100,10 +100,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   int group, rank, g = 0, split = 0, item = 0;
   if (SPLIT) {
     static_assert(!SPLIT || MQ == 1, "split mode maps one row per lane");
-    split = blockIdx.x % p.num_splits;
-    item = blockIdx.x / p.num_splits;
-    rank = p.num_q_tiles - 1 - item % p.num_q_tiles;
-    group = item / p.num_q_tiles;
+    // kv heads vary fastest: in the usual [batch, seq, heads, dim] layout the work-groups dispatched
+    // together then read neighbouring 2 * D bytes of the same key rows at about the same time
+    int r = blockIdx.x;
+    const int kvh = r % p.num_kv_heads;
+    r /= p.num_kv_heads;
+    split = r % p.num_splits;
+    r /= p.num_splits;
+    const int tile = r % p.num_q_tiles;
+    group = (r / p.num_q_tiles) * p.num_kv_heads + kvh;
+    item = group * p.num_q_tiles + tile;
+    rank = p.num_q_tiles - 1 - tile;
   } else {
     const ItemMap items{p.batch * p.num_kv_heads, p.num_q_tiles, p.group};
     if (!items.decode(blockIdx.x, group, rank, g)) return;
