@@ -733,6 +733,14 @@ int launch_dq(BwdParams p, hipStream_t stream) {
 
 template <class Tr, int D>
 int launch_bwd(BwdParams p, hipStream_t stream) {
+  // a key sequence too long for the dQ kernel's largest configuration is refused before anything
+  // is enqueued (the dK/dV kernel has no such limit)
+  if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
+    const int need = DqSmem<D, 3>::kTotal + live_tiles_bytes(8, p.n_kv_tiles);
+    if (need > kLdsPerCu)
+      return fail(KVAX_EUNSUPPORTED, "the dQ kernel needs %d bytes of LDS for tile bitmaps (limit %d): "
+                  "sequence too long", need, kLdsPerCu);
+  }
   // tile summaries of both sequences (a few microseconds; needed by dQ and dK/dV)
   {
     TileSummaryJob jobs[2] = {{p.kv_pos, p.kv_seg, (void*)p.kv_tiles, p.kv_len},

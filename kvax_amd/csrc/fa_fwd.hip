@@ -635,6 +635,13 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
   }
   hipStream_t stream = (hipStream_t)stream_;
   if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
+  {  // too long for the largest configuration: refuse before anything is enqueued
+    const int ring = (2 * kTK * a->head_dim * 2 + 2 * kTK * 4) * 3;
+    const int need = ring + live_tiles_bytes(8, p.n_kv_tiles);
+    if (need > kLdsPerCu)
+      return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
+                  a->kv_len, need, kLdsPerCu);
+  }
   {
     TileSummaryJob job{a->kv_pos, a->kv_seg, workspace, a->kv_len};
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;

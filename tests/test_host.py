@@ -209,3 +209,28 @@ def test_workspace_sizes_follow_the_shapes():
     delta = 1 * 32 * 32768 * 4
     order = (2 * 256 + 1) * 4 + 12                                      # 256 kv work items, padded to 16
     assert bwd(1, 32768, 32768, 32, 8, 128) == delta + 2 * 32 * 512 + order
+
+
+def test_too_long_key_sequences_are_refused_without_a_gpu():
+    """The forward and dQ kernels keep per-tile bitmaps of the key sequence in LDS; a sequence they
+    cannot hold is refused before anything is enqueued (so this runs without a GPU: non-null dummy
+    pointers are never dereferenced)."""
+    lib = _native.lib()
+    a = _fa_args(1, 128, 2_000_000, 8, 2, 128)
+    dummy = 0x1000
+    for field in ("q", "k", "v", "out", "lse", "q_pos", "q_seg", "kv_pos", "kv_seg", "dout", "dq", "dk", "dv"):
+        setattr(a, field, dummy)
+    for name in ("q_strides", "k_strides", "v_strides", "o_strides", "do_strides", "dq_strides",
+                 "dk_strides", "dv_strides"):
+        setattr(a, name, (ctypes.c_int64 * 3)(0, 1024, 128))
+    a.fwd_query_block = a.fwd_kv_block = a.bwd_query_block = a.bwd_kv_block = 128
+    a.dtype, a.scale = _native.KVAX_BF16, 0.1
+    for m in (a.fwd_mask, a.dq_mask, a.dkdv_mask):
+        for i in range(4):
+            m[i] = dummy
+    need = lib.kvax_fa_fwd_workspace_bytes(ctypes.byref(a))
+    assert lib.kvax_fa_fwd(ctypes.byref(a), dummy, need, None) == -2
+    assert b"LDS" in lib.kvax_last_error()
+    need = lib.kvax_fa_bwd_workspace_bytes(ctypes.byref(a))
+    assert lib.kvax_fa_bwd(ctypes.byref(a), dummy, need, None) == -2
+    assert b"LDS" in lib.kvax_last_error()

@@ -286,3 +286,61 @@ def test_strided_views_give_the_same_bits_as_contiguous_tensors(device):
     dense = run(q.contiguous(), k.contiguous(), v.contiguous(), dout.contiguous())
     for name, a, c in zip(("out", "dq", "dk", "dv"), strided, dense):
         assert torch.equal(a, c), name
+
+
+def test_c_abi_rejects_bad_arguments_before_launching(device):
+    """Error paths of kvax_fa_fwd / kvax_fa_bwd with real device pointers: each is reported with its
+    code and a message, and nothing is enqueued (the outputs keep their contents)."""
+    import ctypes as C
+
+    from kvax_amd import _native
+    from kvax_amd.ops.flash_attention import _base_args, _mask_ptrs, _strides3
+
+    lib = _native.lib()
+    data, scale = make_random_attention_inputs(1, 256, 256, 4, 2, 128, 128, seed=2, device=device)
+    q, k, v, *ids = data
+    p = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(*ids, fwd_params=p, bwd_params=p, calc_bwd_mask=True)
+    out = torch.full_like(q, 7.0)
+    lse = torch.zeros(1, 4, 256, dtype=torch.float32, device=device)
+
+    def args():
+        a = _base_args(q, k, v, *ids, scale, p, p)
+        a.out, a.lse, a.o_strides = out.data_ptr(), lse.data_ptr(), _strides3(out)
+        a.fwd_mask = _mask_ptrs(masks[0])
+        return a
+
+    ws = torch.empty(1 << 16, dtype=torch.uint8, device=device)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    fwd = lambda a, w=ws, n=None: lib.kvax_fa_fwd(C.byref(a), w.data_ptr(), w.numel() if n is None else n, stream)
+
+    assert fwd(args()) == 0
+    torch.cuda.synchronize()
+    good = out.clone()
+    out.fill_(7.0)
+
+    a = args()
+    assert fwd(a, n=8) == -3 and b"workspace" in lib.kvax_last_error()                  # too small
+    assert lib.kvax_fa_fwd(C.byref(a), ws.data_ptr() + 4, ws.numel() - 4, stream) == -1  # misaligned
+    a = args(); a.q = q.data_ptr() + 2
+    assert fwd(a) == -1 and b"aligned" in lib.kvax_last_error()
+    a = args(); a.q_strides = (C.c_int64 * 3)(q.stride(0), q.stride(1) + 4, q.stride(2))
+    assert fwd(a) == -1 and b"stride" in lib.kvax_last_error()
+    a = args(); a.k_strides = (C.c_int64 * 3)(k.stride(0), 1 << 24, k.stride(2))
+    assert fwd(a) == -2 and b"stride" in lib.kvax_last_error()
+    a = args(); a.dtype = 5
+    assert fwd(a) == -2
+    a = args(); a.head_dim = 256
+    assert fwd(a) == -2 and b"head_dim" in lib.kvax_last_error()
+    a = args(); a.fwd_query_block = 0
+    assert fwd(a) == -1
+    a = args(); a.flags = 1 << 20
+    assert fwd(a) == -1 and b"flags" in lib.kvax_last_error()
+    a = args(); a.fwd_mask[2] = None
+    assert fwd(a) == -1 and b"mask" in lib.kvax_last_error()
+    # backward: gradient pointers and masks
+    a = args()
+    assert lib.kvax_fa_bwd(C.byref(a), ws.data_ptr(), ws.numel(), stream) == -1
+    assert b"gradient" in lib.kvax_last_error()
+    assert good.abs().max() > 0
