@@ -227,8 +227,14 @@ def main():
                     "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
                     "traffic": recorded_traffic(dominant, args.workload)}
     result = {
-        "metric": "doc-mask attention TFLOP/s, forward+backward, 32k tokens, bf16, unmasked FLOPs"
-                  if backward else "doc-mask attention TFLOP/s, forward, bf16, unmasked FLOPs",
+        # the headline metric's own wording for the configuration it is quoted on; `value` is its
+        # forward+backward figure, the forward one and the mask build time follow as fwd_tflops and
+        # mask_build_ms
+        "metric": "doc-mask attn TFLOP/s fwd & fwd+bwd @32k bf16 (unmasked FLOPs); mask build ms"
+                  if args.workload == "doc32k" else
+                  ("doc-mask attention TFLOP/s, forward+backward, bf16, unmasked FLOPs" if backward
+                   else "doc-mask attention TFLOP/s, forward, bf16, unmasked FLOPs"),
+        "value_is": "forward+backward TFLOP/s" if backward else "forward TFLOP/s",
         "value": value,
         "unit": "TFLOP/s",
         "n_gpus": 1,
