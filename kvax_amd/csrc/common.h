@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "kvax_amd.h"
 
@@ -18,6 +19,35 @@ inline int check_launch(const char* what) {
 }
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// Raises a kernel's dynamic LDS limit once per device, safely under concurrent host threads: the
+// first caller on a device sets the attribute, every caller gets the result of that attempt.  One
+// static instance per kernel instantiation.
+class LdsReservation {
+ public:
+  template <class K>
+  int ensure(K kernel, int bytes, const char* what) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+      return fail(KVAX_ELAUNCH, "cannot identify the current device for %s", what);
+    PerDevice& d = per_device_[dev];
+    std::call_once(d.once, [&] {
+      d.status = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    });
+    if (d.status != hipSuccess)
+      return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for %s: %s", bytes, what,
+                  hipGetErrorString(d.status));
+    return KVAX_OK;
+  }
+
+ private:
+  static constexpr int kMaxDevices = 64;
+  struct PerDevice {
+    std::once_flag once;
+    hipError_t status = hipSuccess;
+  };
+  PerDevice per_device_[kMaxDevices];
+};
 
 // Rows per streamed LDS tile in the attention kernels, and the granularity of the tile summaries.
 constexpr int kTileRows = 64;

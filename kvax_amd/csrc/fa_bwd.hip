@@ -318,6 +318,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   }
 
   if (in) {
+    // Rows that attend to nothing (padding) get exact zeros.  Their accumulator is not zero when the
+    // block mask declares padding-against-padding blocks mask-free (masks built without skipping
+    // padding): the element mask, which is what excludes them, is not applied there.
+    const bool dead = col_width == 0;
     char* row = p.dq + ((int64_t)b * p.dq_sb + (int64_t)head * p.dq_sh + (int64_t)qrow * p.dq_ss) * 2;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
@@ -326,6 +330,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
         uint2 u;
         u.x = Tr::pack2(dq[dt][4 * g4 + 0] * p.scale, dq[dt][4 * g4 + 1] * p.scale);
         u.y = Tr::pack2(dq[dt][4 * g4 + 2] * p.scale, dq[dt][4 * g4 + 3] * p.scale);
+        if (dead) u = make_uint2(0, 0);
         *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
       }
   }
@@ -676,6 +681,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
 
   // ---- epilogue: the P wave holds dV^T, the S wave dK^T (times the scale) ----------------------
   if (in) {
+    const bool dead = col_width == 0;  // padding keys: exact zeros (see the dQ kernel's epilogue)
     const float mul = p_wave ? 1.f : p.scale;
     char* base = p_wave ? p.dv : p.dk;
     const int64_t sb = p_wave ? p.dv_sb : p.dk_sb, sh = p_wave ? p.dv_sh : p.dk_sh, ss = p_wave ? p.dv_ss : p.dk_ss;
@@ -687,8 +693,9 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++)
           *reinterpret_cast<float4*>(row + 32 * dt + 8 * g4 + 4 * h) =
-              make_float4(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul, acc[dt][4 * g4 + 2] * mul,
-                          acc[dt][4 * g4 + 3] * mul);
+              dead ? make_float4(0.f, 0.f, 0.f, 0.f)
+                   : make_float4(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul,
+                                 acc[dt][4 * g4 + 2] * mul, acc[dt][4 * g4 + 3] * mul);
     } else {
       char* row = base + off * 2;
 #pragma unroll
@@ -698,6 +705,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
           uint2 u;
           u.x = Tr::pack2(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul);
           u.y = Tr::pack2(acc[dt][4 * g4 + 2] * mul, acc[dt][4 * g4 + 3] * mul);
+          if (dead) u = make_uint2(0, 0);
           *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
         }
     }
@@ -705,23 +713,18 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
 }
 
 template <class K>
-int reserve_lds(K kernel, int need, int bytes, bool* done, const char* what) {
+int reserve_lds(K kernel, int need, int bytes, LdsReservation* reservation, const char* what) {
   if (need > bytes)
     return fail(KVAX_EUNSUPPORTED, "%s needs %d bytes of LDS for tile bitmaps (limit %d): sequence too long",
                 what, need, bytes);
-  if (*done) return KVAX_OK;
-  if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) !=
-      hipSuccess)
-    return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for %s", bytes, what);
-  *done = true;
-  return KVAX_OK;
+  return reservation->ensure(kernel, bytes, what);
 }
 
 // dQ launch: NW wavefronts (32 query rows each) per work-group, two per SIMD.
 template <class Tr, int D, int NW, int STAGES>
 int launch_dq(BwdParams p, hipStream_t stream) {
   auto kernel = fa_bwd_dq_kernel<Tr, D, NW, 2, STAGES>;
-  static bool done = false;
+  static LdsReservation done;
   constexpr int kLimit = kLdsPerCu / (8 / NW);
   const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   if (int rc = reserve_lds(kernel, smem, kLimit, &done, "the dQ kernel")) return rc;
@@ -778,7 +781,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   if (run_dkdv) {
     constexpr int NW = 8;
     auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2>;
-    static bool done = false;
+    static LdsReservation done;
     // live-tile bookkeeping for as many query tiles as the remaining LDS holds (a multiple of 64)
     constexpr int kLdsLimit = kLdsPerCu;
     int chunk = 64;

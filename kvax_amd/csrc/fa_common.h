@@ -274,6 +274,10 @@ __device__ __forceinline__ int swz(int r) {
 // (wave-uniform), lane i providing its own global source address.  Completion is tracked by
 // vmcnt; the data is visible to other waves after an s_waitcnt vmcnt + barrier.  Issued through
 // inline assembly so that the compiler does not serialise later LDS reads against it.
+// The statements write M0 without naming it as a clobber: M0 is a reserved register for this
+// target (clang rejects it in a clobber list with a warning and ignores it), the compiler never
+// keeps a value live in it and loads it immediately before each use of its own (indirect register
+// indexing, s_sendmsg, its LDS-DMA builtins) - none of which these kernels contain.
 __device__ __forceinline__ void async_copy_b128(const void* gptr, uint32_t lds_addr) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(gptr)
                : "memory");

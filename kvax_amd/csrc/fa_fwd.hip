@@ -513,13 +513,8 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   if (smem > kMaxSmem)
     return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
                 p.kv_len, smem, kMaxSmem);
-  static bool configured = false;  // benign race: the attribute is idempotent
-  if (!configured) {
-    if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kMaxSmem) != hipSuccess)
-      return fail(KVAX_ELAUNCH, "cannot reserve %d bytes of LDS for the forward kernel", kMaxSmem);
-    configured = true;
-  }
+  static LdsReservation reservation;  // one per instantiation of this function template
+  if (int rc = reservation.ensure(kernel, kMaxSmem, "the forward kernel")) return rc;
   hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
   if (int rc = check_launch("fa_fwd_kernel")) return rc;
   if (SPLIT && p.num_splits > 1) {

@@ -262,6 +262,13 @@ def flash_attention(
     """Attention over packed documents with a block-sparse mask.
 
     Arguments and defaults as in the reference (flash_attention_triton.py:2027-2095).
+
+    Precondition on the ids (the reference's too): along every sequence the documents lie one after
+    another, i.e. a segment id never comes back once another id has followed it (``0 0 1 1 2`` is
+    fine, ``0 1 0`` is not; padding, id -1, may sit anywhere).  The block mask's mask-free range
+    ``[lower_full, upper_full)`` is computed from per-block id extremes and is only right for such
+    layouts; the kernels trust it, so ids that return to an earlier value give wrong results
+    without an error.  Ids need not be sorted or dense (``5 5 2 2 7`` is fine).
     Query/key head dims 16, 32, 64, 128 and any value head dim up to 128 are taken (the kernels run
     at 64 or 128; other sizes are zero-padded here).
     ``memory_optimized_gqa_backward`` is accepted and has no effect: dK/dV are always reduced

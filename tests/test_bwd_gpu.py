@@ -1,12 +1,12 @@
 """Backward parity of the HIP flash-attention kernels (through the C ABI and the autograd
 wrapper) with the dense CPU oracle.
 
-Tolerance: max abs error <= 2e-2 on dQ, dK, dV (the build's target).  Two refinements where the
-number format, not the kernel, sets the floor: (1) for |gradient| >= 2 a bf16 result rounds by up
-to 7.8e-3..3.1e-2, so the reference's relative bound is added above 2 (rtol 1e-2 for dQ, 3e-2 for
-dK/dV, kvax/utils/benchmarking.py:614-627); (2) dK/dV are additionally checked as fp32 (the
-reference kernels' own output type) against the plain 2e-2 bound in
-``test_fp32_dkdv_within_plain_bound``.
+Tolerance: max abs error <= 2e-2 on dQ, dK, dV (the build's target) plus the rounding of the
+output format, half a unit in the last place of a 16-bit result (``tests/tolerances.py``); the
+reference's own bounds are atol 3e-2 with rtol 1e-2 (dQ) / 3e-2 (dK, dV),
+kvax/utils/benchmarking.py:614-627.  dK/dV are additionally checked as fp32 (the reference
+kernels' own output type) against the plain 2e-2, on small cases and on the sampled GQA group of
+the full-size workloads.  Every check prints the largest error it saw (``pytest -s`` shows them).
 """
 import numpy as np
 import pytest
@@ -20,10 +20,10 @@ from kvax_amd.utils.benchmarking import (
     workload,
 )
 from oracle import attention_oracle as ao
+from tests.tolerances import ATOL, check_close
 
 pytestmark = pytest.mark.gpu
 TP_SPECS = (("data", None, "model", None), ("data", None, "model", None))
-ATOL = 2e-2
 
 
 def run_backward(data, scale, fwd_blocks, bwd_blocks, dout):
@@ -48,21 +48,17 @@ def oracle_backward(data, scale, dout, heads=None, dtype=np.float64, row_block=4
                                  row_block=row_block)
 
 
-def check_grad(name, got, ref, rtol, atol=ATOL):
-    got = got.float().cpu().numpy()
-    assert np.isfinite(got).all(), name
-    err = np.abs(got - ref)
-    bound = atol + rtol * np.maximum(np.abs(ref) - 2.0, 0.0)
-    worst = (err - bound).max()
-    assert worst <= 0, f"{name}: max abs err {err.max():.4g} (|ref| max {np.abs(ref).max():.3g})"
-    return err.max()
+def check_grad(name, got, ref, atol=ATOL):
+    worst = check_close(name, got, ref, atol)
+    print(f"    {name}: max abs err {worst:.3e} (|ref| max {np.abs(ref).max():.3g})")
+    return worst
 
 
 def check_all(grads, refs, q_seg, kv_seg, kv_atol=ATOL):
     dq, dk, dv = grads
-    check_grad("dq", dq, refs[0], 1e-2)
-    check_grad("dk", dk, refs[1], 3e-2, kv_atol)
-    check_grad("dv", dv, refs[2], 3e-2, kv_atol)
+    check_grad("dq", dq, refs[0])
+    check_grad("dk", dk, refs[1], kv_atol)
+    check_grad("dv", dv, refs[2], kv_atol)
     qpad = q_seg.cpu().numpy() == -1
     kpad = kv_seg.cpu().numpy() == -1
     assert (dq.float().cpu().numpy()[qpad] == 0).all(), "padding rows of dQ must be zero"
@@ -139,9 +135,8 @@ def test_fp32_dkdv_within_plain_bound(device, case):
                                           out, lse, dout, scale, fwd, bwd, dkdv_fp32=True)
     assert dk.dtype == torch.float32 and dv.dtype == torch.float32
     refs = oracle_backward(data, scale, dout)
-    for name, got, ref in (("dk", dk, refs[1]), ("dv", dv, refs[2])):
-        err = np.abs(got.cpu().numpy() - ref).max()
-        assert err <= ATOL, f"{name}: max abs err {err:.4g}"
+    for name, got, ref in (("dk fp32", dk, refs[1]), ("dv fp32", dv, refs[2])):
+        check_grad(name, got, ref)
 
 
 def test_backward_fp16(device):
@@ -175,21 +170,112 @@ def test_gqa_equals_repeated_kv_heads(device):
     assert (dv.float() - dv2).abs().max().item() <= 3e-2
 
 
-@pytest.mark.parametrize("name, heads", [("doc32k", [8, 9, 10, 11]), ("block_skip", [56, 57, 58, 59, 60, 61, 62, 63])])
-def test_measurement_workloads_sampled_group(device, name, heads):
-    """Full-size configurations.  The oracle evaluates one whole GQA group so that dK/dV of its kv
-    head are complete; dQ is checked on those heads."""
-    w = workload(name)
+_GROUP_ORACLE = {}
+
+
+def _sampled_group_oracle(name, heads):
+    """Oracle gradients of one GQA group of a full-size workload (batch row 0), computed once per
+    process: they do not depend on the mask block size."""
+    if name not in _GROUP_ORACLE:
+        w = workload(name)
+        q, k, v, dout = w.draw_tensors(0, "cpu", with_dout=True)
+        data = tuple(x[:1] for x in (q, k, v) + w.ids("cpu"))
+        _GROUP_ORACLE[name] = oracle_backward(data, w.scale, dout[:1], heads=heads, dtype=np.float32,
+                                              row_block=2048)
+    return _GROUP_ORACLE[name]
+
+
+@pytest.mark.parametrize("name, block, heads", [
+    ("doc32k", 128, [8, 9, 10, 11]),
+    ("block_skip", 128, [56, 57, 58, 59, 60, 61, 62, 63]),
+    ("block_skip", 64, [56, 57, 58, 59, 60, 61, 62, 63]),
+])
+def test_measurement_workloads_sampled_group(device, name, block, heads):
+    """Full-size configurations at every mask block size they are specified for.  The oracle
+    evaluates one whole GQA group so that dK/dV of its kv head are complete; dQ is checked on those
+    heads.  Two runs: the public op (16-bit gradients, bound = 2e-2 + output rounding) and the C ABI
+    with fp32 dK/dV (plain 2e-2)."""
+    from kvax_amd.ops.flash_attention import flash_attention_backward, flash_attention_forward
+
+    w = workload(name, block=block)
     q, k, v, dout = w.draw_tensors(0, device, with_dout=True)
-    data = (q, k, v) + w.ids(device)
+    ids = w.ids(device)
+    data = (q, k, v) + ids
     _, dq, dk, dv = run_backward(data, w.scale, w.fwd_blocks, w.bwd_blocks, dout)
+    refs = _sampled_group_oracle(name, heads)
     b = slice(0, 1)
-    refs = oracle_backward(tuple(x[b] for x in data), w.scale, dout[b], heads=heads,
-                           dtype=np.float32, row_block=2048)
     kvh = heads[0] // (w.num_heads // w.num_kv_heads)
-    check_grad("dq", dq[b][:, :, heads], refs[0][:, :, heads], 1e-2)
-    check_grad("dk", dk[b][:, :, kvh], refs[1][:, :, kvh], 3e-2)
-    check_grad("dv", dv[b][:, :, kvh], refs[2][:, :, kvh], 3e-2)
+    print(f"  {name} block {block}, public op:")
+    check_grad("dq", dq[b][:, :, heads], refs[0][:, :, heads])
+    check_grad("dk", dk[b][:, :, kvh], refs[1][:, :, kvh])
+    check_grad("dv", dv[b][:, :, kvh], refs[2][:, :, kvh])
+    del dq, dk, dv
+    fp, bp = FlashAttentionParamsConfig(*w.fwd_blocks), FlashAttentionParamsConfig(*w.bwd_blocks)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(*ids, fwd_params=fp, bwd_params=bp, calc_bwd_mask=True)
+    out, lse = flash_attention_forward(q, k, v, *ids, masks[0], w.scale, fp, bp)
+    _, dk32, dv32 = flash_attention_backward(q, k, v, *ids, masks[1], masks[2], out, lse, dout, w.scale,
+                                             fp, bp, dkdv_fp32=True)
+    assert dk32.dtype == torch.float32 and dv32.dtype == torch.float32
+    print(f"  {name} block {block}, fp32 dK/dV:")
+    check_grad("dk fp32", dk32[b][:, :, kvh], refs[1][:, :, kvh])
+    check_grad("dv fp32", dv32[b][:, :, kvh], refs[2][:, :, kvh])
+
+
+@pytest.mark.parametrize("hq, hkv, d", [(4, 2, 128), (8, 1, 64)])
+def test_negative_scale(device, hq, hkv, d):
+    """A negative scale is folded into the operands three different ways (Q negated in the forward,
+    a signed exponent scale in dQ, K negated in dK/dV); all must agree with the oracle."""
+    data, scale = make_random_attention_inputs(2, 640, 640, hq, hkv, d, d, seed=11, num_pad_tokens=90,
+                                               list_of_segment_lengths=[200, 250, -1], device=device)
+    scale = -scale
+    dout = torch.randn(data[0].shape, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).to(device)
+    out, dq, dk, dv = run_backward(data, scale, (64, 64), (64, 128), dout)
+    q_, k_, v_, *ids_ = [x.cpu() for x in data]
+    ref_out, _ = ao.attention_forward(q_.float().numpy(), k_.float().numpy(), v_.float().numpy(),
+                                      *[x.numpy() for x in ids_], scale)
+    check_grad("out", out, ref_out)
+    # sanity of the case itself: the sign matters (softmax(-s) differs from softmax(s))
+    pos_out, _ = ao.attention_forward(q_.float().numpy(), k_.float().numpy(), v_.float().numpy(),
+                                      *[x.numpy() for x in ids_], -scale)
+    assert np.abs(pos_out - ref_out).max() > 0.1
+    check_all((dq, dk, dv), oracle_backward(data, scale, dout), data[4], data[6],
+              kv_atol=5e-2 if hkv == 1 else ATOL)
+
+
+@pytest.mark.parametrize("restart", [False, True])
+def test_masks_built_without_skipping_padding(device, restart):
+    """With ``skip_pad_tokens=False`` the block mask treats padding like one more document (blocks of
+    padding against padding are 'full'); the attention kernels must still give padding rows zeros
+    and the other rows the oracle's values."""
+    w = workload("doc32k", restart_positions=restart)
+    n = 4096  # a prefix of the 32k layout: several documents, then padding is appended
+    q_pos, q_seg = w.q_pos[:, :n].copy(), w.q_seg[:, :n].copy()
+    q_seg[:, n - 700:] = -1
+    q_pos[:, n - 700:] = np.arange(700) if restart else np.arange(n - 700, n)
+    g = torch.Generator().manual_seed(21)
+    q = torch.randn((1, n, 8, 128), generator=g).to(torch.bfloat16).to(device)
+    k = torch.randn((1, n, 2, 128), generator=g).to(torch.bfloat16).to(device)
+    v = torch.randn((1, n, 2, 128), generator=g).to(torch.bfloat16).to(device)
+    dout = torch.randn((1, n, 8, 128), generator=g).to(torch.bfloat16).to(device)
+    ids = tuple(torch.from_numpy(x).to(device) for x in (q_pos, q_seg, q_pos, q_seg))
+    scale = 128 ** -0.5
+    qg, kg, vg = (x.clone().requires_grad_(True) for x in (q, k, v))
+    params = FlashAttentionParamsConfig(128, 128)
+    with attention_specs(*TP_SPECS):
+        masks = create_attention_mask(*ids, fwd_params=params, bwd_params=params, calc_bwd_mask=True,
+                                      skip_pad_tokens=False)
+        skipping = create_attention_mask(*ids, fwd_params=params, bwd_params=params, calc_bwd_mask=True)
+        out = flash_attention(qg, kg, vg, *ids, masks, scale=scale, fwd_params=params, bwd_params=params)
+    # the case must differ from the default masks: padding blocks are visited here
+    assert not torch.equal(masks[0].upper_bounds, skipping[0].upper_bounds)
+    out.backward(dout)
+    data = (q, k, v) + ids
+    ref_out, _ = ao.attention_forward(q.float().cpu().numpy(), k.float().cpu().numpy(),
+                                      v.float().cpu().numpy(), q_pos, q_seg, q_pos, q_seg, scale)
+    check_grad("out", out, ref_out)
+    assert (out.detach().float().cpu().numpy()[q_seg == -1] == 0).all()
+    check_all((qg.grad, kg.grad, vg.grad), oracle_backward(data, scale, dout), ids[1], ids[3])
 
 
 def test_missing_backward_masks(device):

@@ -18,12 +18,14 @@ from kvax_amd import (
     permute_tokens_context_parallelism,
     unpermute_tokens_context_parallelism,
 )
+from kvax_amd.ops.flash_attention import flash_attention_backward, flash_attention_forward
 from kvax_amd.utils.benchmarking import (
     generate_random_segments_lengths,
     make_random_attention_inputs,
     workload,
 )
 from oracle import attention_oracle as ao
+from tests.tolerances import check_close
 
 pytestmark = pytest.mark.gpu
 TP_SPECS = (("data", None, "model", None), ("data", None, "model", None))
@@ -110,13 +112,19 @@ def test_cp_shard_workload_against_oracle(device, rank):
     args = (f(q), f(k), f(v), w.q_pos, w.q_seg, w.kv_pos, w.kv_seg, w.scale)
     ref_out, _ = ao.attention_forward(*args, dtype=np.float32, heads=heads, row_block=1024)
     ref_dq, ref_dk, ref_dv = ao.attention_backward(*args, f(dout), dtype=np.float32, heads=heads, row_block=1024)
-    def ok(name, got, ref, rtol):
-        err = np.abs(got - ref)
-        assert (err <= 2e-2 + rtol * np.maximum(np.abs(ref) - 2.0, 0)).all(), f"{name}: {err.max()}"
-    ok("out", f(out)[:, :, heads], ref_out[:, :, heads], 0.0)
-    ok("dq", f(q.grad)[:, :, heads], ref_dq[:, :, heads], 1e-2)
-    ok("dk", f(k.grad)[:, :, 1], ref_dk[:, :, 1], 3e-2)
-    ok("dv", f(v.grad)[:, :, 1], ref_dv[:, :, 1], 3e-2)
+    # 2e-2 plus the rounding of the 16-bit result (tests/tolerances.py)
+    worst = {"out": check_close("out", out[:, :, heads], ref_out[:, :, heads]),
+             "dq": check_close("dq", q.grad[:, :, heads], ref_dq[:, :, heads]),
+             "dk": check_close("dk", k.grad[:, :, 1], ref_dk[:, :, 1]),
+             "dv": check_close("dv", v.grad[:, :, 1], ref_dv[:, :, 1])}
+    # dK/dV of the sampled kv head straight from the fp32 accumulators: plain 2e-2
+    with torch.no_grad():
+        out2, lse = flash_attention_forward(q, k, v, *ids, masks[0], w.scale, fp, bp)
+        _, dk32, dv32 = flash_attention_backward(q, k, v, *ids, masks[1], masks[2], out2, lse, dout,
+                                                 w.scale, fp, bp, dkdv_fp32=True)
+    worst["dk fp32"] = check_close("dk fp32", dk32[:, :, 1], ref_dk[:, :, 1])
+    worst["dv fp32"] = check_close("dv fp32", dv32[:, :, 1], ref_dv[:, :, 1])
+    print(f"  cp_shard rank {rank}: " + ", ".join(f"{n} {e:.3e}" for n, e in worst.items()))
 
 
 @pytest.mark.parametrize("heads, kv_heads, batch", [(6, 3, 1), (4, 2, 1), (2, 1, 1), (8, 8, 3)])
@@ -130,7 +138,6 @@ def test_work_distribution_modes(device, heads, kv_heads, batch):
     args = tuple(f(x) if x.dtype == torch.bfloat16 else x.cpu().numpy() for x in data) + (scale,)
     ref_out, _ = ao.attention_forward(*args)
     ref = ao.attention_backward(*args, f(dout))
-    assert np.abs(f(out) - ref_out).max() <= 2e-2
-    for got, want, rtol in zip((dq, dk, dv), ref, (1e-2, 3e-2, 3e-2)):
-        err = np.abs(f(got) - want)
-        assert (err <= 2e-2 + rtol * np.maximum(np.abs(want) - 2.0, 0)).all(), err.max()
+    check_close("out", out, ref_out)
+    for name, got, want in zip(("dq", "dk", "dv"), (dq, dk, dv), ref):
+        check_close(name, got, want)

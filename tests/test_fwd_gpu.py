@@ -170,21 +170,49 @@ def test_constant_positions_are_bidirectional(device):
     assert (out - ref).abs().max().item() <= ATOL
 
 
-@pytest.mark.parametrize("name, heads", [("dense_causal", [0, 13]), ("doc32k", [5]),
-                                         ("block_skip", [0, 63])])
-def test_measurement_workloads_sampled_heads(device, name, heads):
-    """Full-size configurations; the dense oracle is evaluated for a sample of heads only."""
-    w = workload(name)
+_HEADS_ORACLE = {}
+
+
+def _sampled_heads_oracle(name, heads):
+    """Oracle output of a few heads of a full-size workload (batch row 0), computed once per
+    process: it does not depend on the mask block size."""
+    if name not in _HEADS_ORACLE:
+        w = workload(name)
+        q, k, v = w.draw_tensors(0, "cpu", with_dout=False)
+        ref, _ = ao.attention_forward(q[:1].float().numpy(), k[:1].float().numpy(), v[:1].float().numpy(),
+                                      w.q_pos[:1], w.q_seg[:1], w.kv_pos[:1], w.kv_seg[:1],
+                                      w.scale, dtype=np.float32, heads=heads, row_block=2048)
+        _HEADS_ORACLE[name] = ref
+    return _HEADS_ORACLE[name]
+
+
+@pytest.mark.parametrize("name, block, heads", [("dense_causal", 128, [0, 13]), ("doc32k", 128, [5]),
+                                                ("block_skip", 128, [0, 63]), ("block_skip", 64, [0, 63])])
+def test_measurement_workloads_sampled_heads(device, name, block, heads):
+    """Full-size configurations at every mask block size they are specified for; the dense oracle is
+    evaluated for a sample of heads of the first batch row."""
+    w = workload(name, block=block)
     q, k, v = w.draw_tensors(0, device, with_dout=False)
     data = (q, k, v) + w.ids(device)
+    assert w.fwd_blocks == (block, block)
     out = run_forward(data, w.scale, *w.fwd_blocks)
-    b = slice(0, 1)  # first batch row is enough for the oracle
-    small = tuple(x[b] for x in data)
-    q_, k_, v_, q_pos, q_seg, kv_pos, kv_seg = [x.cpu() for x in small]
-    ref, _ = ao.attention_forward(q_.float().numpy(), k_.float().numpy(), v_.float().numpy(),
-                                  q_pos.numpy(), q_seg.numpy(), kv_pos.numpy(), kv_seg.numpy(),
-                                  w.scale, dtype=np.float32, heads=heads, row_block=2048)
-    check(out[b], ref, q_seg, heads=heads)
+    check(out[:1], _sampled_heads_oracle(name, heads), data[4][:1], heads=heads)
+
+
+def test_unsorted_document_ids(device):
+    """Documents laid out one after another whose ids are neither sorted nor dense (9, 2, 5 ...):
+    allowed; only an id that comes back after another one is outside the contract."""
+    data, scale = make_random_attention_inputs(2, 1024, 1024, 4, 2, 128, 128, seed=17, num_pad_tokens=120,
+                                               list_of_segment_lengths=[200, 130, 300, 64, -1],
+                                               device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    relabel = torch.tensor([9, 2, 5, 1000000, 3], dtype=torch.int32, device=device)
+    q_seg = torch.where(q_seg == -1, q_seg, relabel[q_seg.clamp(min=0).long()])
+    kv_seg = torch.where(kv_seg == -1, kv_seg, relabel[kv_seg.clamp(min=0).long()])
+    data = (q, k, v, q_pos, q_seg, kv_pos, kv_seg)
+    for block in (64, 128):
+        out = run_forward(data, scale, block, block)
+        check(out, oracle_forward(data, scale), q_seg)
 
 
 def test_errors(device):

@@ -7,7 +7,8 @@ from kvax_amd.ops.mask_creator import build_masks, create_attention_mask
 from kvax_amd.utils import FlashAttentionParamsConfig, Mesh, attention_specs
 from kvax_amd.utils.benchmarking import workload
 from oracle import mask_oracle as mo
-from tests.test_oracle_mask import REFERENCE_MASK_CASES, _random_ids, reference_mask_case
+from tests.test_oracle_mask import (REFERENCE_MASK_CASES, STYLE_SEEDS, _random_ids,
+                                     hand_worked_mask_cases, reference_mask_case)
 
 pytestmark = pytest.mark.gpu
 
@@ -30,7 +31,7 @@ def _assert_masks_equal(got, want):
 @pytest.mark.parametrize("style", ["restart", "global", "unsorted", "shuffled_pos"])
 @pytest.mark.parametrize("skip_pad", [True, False])
 def test_random_ragged_inputs(device, style, skip_pad):
-    rng = np.random.default_rng(hash((style, skip_pad, "gpu")) % 2**32)
+    rng = np.random.default_rng([STYLE_SEEDS[style], int(skip_pad), 7])
     for trial in range(10):
         batch = int(rng.integers(1, 4))
         sq = int(rng.integers(1, 700))
@@ -44,6 +45,15 @@ def test_random_ragged_inputs(device, style, skip_pad):
                 mo.block_mask_c(q_pos, q_seg, kv_pos, kv_seg, kbs, qbs, skip_pad, False),
                 mo.block_mask_c(q_pos, q_seg, kv_pos, kv_seg, qbs, kbs, skip_pad, True)]
         _assert_masks_equal(got, want)
+
+
+@pytest.mark.parametrize("ids, m", hand_worked_mask_cases())
+def test_hand_worked_vectors(device, ids, m):
+    """Expected arrays derived on paper from the reference's kernel (tests/golden)."""
+    got = build_masks(*_dev(device, *ids), [(m["query_block"], m["kv_block"], m["kv_outer"])],
+                      m["skip_pad"])[0]
+    for name, x in zip(("lower", "upper", "lower_full", "upper_full"), got.flatten()):
+        np.testing.assert_array_equal(x.cpu().numpy()[0, 0], np.asarray(m[name], np.int32), err_msg=name)
 
 
 @pytest.mark.parametrize("case", REFERENCE_MASK_CASES)
