@@ -147,6 +147,19 @@ int kvax_fa_fwd(const kvax_fa_args* args, void* workspace, size_t workspace_byte
 int kvax_fa_bwd(const kvax_fa_args* args, void* workspace, size_t workspace_bytes,
                 kvax_stream_t stream);
 
+/* kvax_fa_fwd without a workspace argument, for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (there XLA owns every buffer).  Same arguments, kernels and results
+ * as kvax_fa_fwd; the scratch memory is a buffer of KVAX_FA_FWD_STATIC_MAX_WORKSPACE bytes that the
+ * library holds in device memory on every GPU it runs on until the process ends.  A call whose
+ * kvax_fa_fwd_workspace_bytes() exceeds that size fails with KVAX_EWORKSPACE and enqueues nothing
+ * (long key sequences in split mode are the only such case: 8 MiB cover 32 rows x 32 query heads
+ * decoding against 128k keys).  The call allocates and frees nothing and does not synchronise.
+ * All calls on one GPU share the buffer: calls that overlap in time on one GPU (different streams
+ * or host threads) race; serialise them or use kvax_fa_fwd with separate workspaces. */
+#define KVAX_FA_FWD_STATIC_MAX_WORKSPACE (8u << 20)
+int kvax_fa_fwd_static(const kvax_fa_args* args, kvax_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,6 +15,7 @@ KVAX_MAX_MASKS = 4
 KVAX_BF16, KVAX_F16 = 0, 1
 KVAX_FA_DKDV_F32 = 1
 KVAX_FA_SKIP_DELTA, KVAX_FA_SKIP_DQ, KVAX_FA_SKIP_DKDV = 16, 32, 64
+KVAX_FA_FWD_STATIC_MAX_WORKSPACE = 8 << 20
 
 
 class KvaxNativeError(RuntimeError):
@@ -90,6 +91,9 @@ def lib() -> C.CDLL:
             fn = getattr(l, name)
             fn.restype = C.c_int
             fn.argtypes = [C.POINTER(FaArgs), C.c_void_p, C.c_size_t, C.c_void_p]
+    if hasattr(l, "kvax_fa_fwd_static"):
+        l.kvax_fa_fwd_static.restype = C.c_int
+        l.kvax_fa_fwd_static.argtypes = [C.POINTER(FaArgs), C.c_void_p]
     for name in ("kvax_fa_fwd_workspace_bytes", "kvax_fa_bwd_workspace_bytes"):
         if hasattr(l, name):
             fn = getattr(l, name)

@@ -580,12 +580,64 @@ extern "C" size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* a) {
   return tile_summary_bytes(a->batch, a->kv_len) + plan.part_o_bytes + plan.part_ml_bytes;
 }
 
+// Scratch memory of kvax_fa_fwd_static: one copy per GPU the library runs on, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress(); the device
+// address it yields is what kernels and memory operations are given.
+constexpr size_t kStaticScratchBytes = KVAX_FA_FWD_STATIC_MAX_WORKSPACE;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** ptr) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mutex;
+  static void* address[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(KVAX_ELAUNCH, "cannot identify the current device");
+  std::lock_guard<std::mutex> lock(mutex);
+  if (!address[dev]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(KVAX_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+    address[dev] = p;
+  }
+  *ptr = address[dev];
+  return KVAX_OK;
+}
+
+int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, kvax_stream_t stream_);
+
+}  // namespace
+
 extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
                            kvax_stream_t stream_) {
   if (int rc = validate_fa_common(a)) return rc;
   const size_t need = kvax_fa_fwd_workspace_bytes(a);
   if (need > workspace_bytes || (need && !workspace))
     return fail(KVAX_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  return fa_fwd_impl(a, workspace, workspace_bytes, stream_);
+}
+
+extern "C" int kvax_fa_fwd_static(const kvax_fa_args* a, kvax_stream_t stream_) {
+  if (int rc = validate_fa_common(a)) return rc;
+  const size_t need = kvax_fa_fwd_workspace_bytes(a);
+  if (need > kStaticScratchBytes)
+    return fail(KVAX_EWORKSPACE, "this call needs %zu bytes of scratch memory, the library's static "
+                "buffer holds %zu: use kvax_fa_fwd with a caller-provided workspace", need,
+                kStaticScratchBytes);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // Nothing in the buffer has to start at zero: the tile summaries and, in split mode, every
+  // partial result that is read are written by this call's own kernels first.
+  return fa_fwd_impl(a, ws, kStaticScratchBytes, stream_);
+}
+
+namespace {
+int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, kvax_stream_t stream_) {
+  (void)workspace_bytes;
   if ((uintptr_t)workspace % 16) return fail(KVAX_EINVAL, "workspace must be 16-byte aligned");
   if (a->fwd_query_block <= 0 || a->fwd_kv_block <= 0)
     return fail(KVAX_EINVAL, "forward block sizes must be positive");
@@ -646,3 +698,4 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
     return bf16 ? launch_fwd_auto<Bf16, 128>(p, stream) : launch_fwd_auto<F16, 128>(p, stream);
   return bf16 ? launch_fwd_auto<Bf16, 64>(p, stream) : launch_fwd_auto<F16, 64>(p, stream);
 }
+}  // namespace

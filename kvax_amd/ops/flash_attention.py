@@ -106,9 +106,11 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
 
 
 def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd_mask, scale,
-                            fwd_params, bwd_params, buffers=None):
+                            fwd_params, bwd_params, buffers=None, static_scratch=False):
     """One device's forward: returns (out like query, lse fp32 [batch, heads, q_len]).
-    ``buffers`` = (out, lse) lets a caller reuse its output tensors."""
+    ``buffers`` = (out, lse) lets a caller reuse its output tensors.  With ``static_scratch`` (and
+    ``buffers``) the call goes through ``kvax_fa_fwd_static`` and allocates no device memory: the
+    scratch memory is the library's own fixed buffer, shared by all calls on the GPU."""
     b, sq, hq, d = query.shape
     if buffers is not None:
         out, lse = buffers
@@ -119,6 +121,12 @@ def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd
     a.out, a.lse, a.o_strides = out.data_ptr(), lse.data_ptr(), _strides3(out)
     a.fwd_mask = _mask_ptrs(fwd_mask)
     lib = _native.lib()
+    if static_scratch:
+        with torch.cuda.device(query.device):
+            stream = torch.cuda.current_stream().cuda_stream
+            rc = lib.kvax_fa_fwd_static(C.byref(a), C.c_void_p(stream))
+        _native.check(rc, "kvax_fa_fwd_static")
+        return out, lse
     ws = _workspace(lib.kvax_fa_fwd_workspace_bytes(C.byref(a)), query.device)
     with torch.cuda.device(query.device):
         stream = torch.cuda.current_stream().cuda_stream
