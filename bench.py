@@ -7,6 +7,9 @@ A step is one forward + backward pass of document-mask attention over one batch 
 synthetic tensors that already live in HBM, through the C ABI (kvax_fa_fwd, kvax_fa_bwd).  The
 block masks are built once before the loop, as a training step would build them once per batch
 and reuse them across layers; their build time is reported separately (``mask_build_ms``).
+After the headline workload (doc32k) the other configurations of the baseline - dense causal forward,
+the context-parallel shard, the block-skipping case at mask blocks 128 and 64, and a decoding step -
+are timed for a few steps each and reported under ``other_workloads`` of the same line.
 Prints ONE JSON line.  ``value`` counts only unmasked FLOPs: 4*D per attendable (q, kv) pair
 and query head in the forward, 2.5x that in the backward.
 """
@@ -64,6 +67,9 @@ def parse():
     ap.add_argument("--block", type=int, default=128)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="skip the brief timing of the other configurations (other_workloads)")
+    ap.add_argument("--secondary-steps", type=int, default=10)
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run a plain streaming kernel of known size (reads and writes "
                          f"{CALIBRATION_BYTES >> 20} MiB) so that a rocprofv3 --pmc run of this command "
@@ -109,25 +115,25 @@ def cpu_baseline(w, seed, seconds_hint=20.0):
     }
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path has no "
-              "collectives.  Run with --gpus 1.", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
+def measure(args, name, block, steps, warmup, device_tensors=False):
+    """Times `steps` forward(+backward) passes of one workload; returns (workload, dict of figures).
+    device_tensors: draw Q/K/V/dO on the GPU (seeded) instead of on the host - same distribution,
+    much faster for the large secondary workloads, whose values do not matter for timing."""
     from kvax_amd import FlashAttentionParamsConfig, _native, attention_specs, create_attention_mask
     from kvax_amd.ops.flash_attention import (backward_workspace_bytes, flash_attention_backward,
                                               flash_attention_forward)
     from kvax_amd.utils.benchmarking import workload
 
     dev = torch.device("cuda:0")
-    w = workload(args.workload, seed=args.seed, restart_positions=not args.global_positions,
-                 block=args.block)
-    tensors = w.draw_tensors(args.seed, dev, with_dout=True)
-    q, k, v, dout = tensors
+    w = workload(name, seed=args.seed, restart_positions=not args.global_positions, block=block)
+    if device_tensors:
+        g = torch.Generator(device=dev).manual_seed(args.seed)
+        shape_q = (w.batch, w.q_len, w.num_heads, w.head_dim)
+        shape_k = (w.batch, w.kv_len, w.num_kv_heads, w.head_dim)
+        q, k, v, dout = (torch.randn(sh, generator=g, device=dev, dtype=torch.float32).to(w.dtype)
+                         for sh in (shape_q, shape_k, shape_k, shape_q))
+    else:
+        q, k, v, dout = w.draw_tensors(args.seed, dev, with_dout=True)
     decode = w.q_len == 1
     ids = w.ids(dev)
     fp, bp = FlashAttentionParamsConfig(*w.fwd_blocks), FlashAttentionParamsConfig(*w.bwd_blocks)
@@ -158,7 +164,7 @@ def main():
     lse = torch.empty((w.batch, w.num_heads, w.q_len), dtype=torch.float32, device=dev)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     ws = torch.empty(backward_workspace_bytes(q, k) + 16, dtype=torch.uint8, device=dev)
-    SD, SQ, SK = _native.KVAX_FA_SKIP_DELTA, _native.KVAX_FA_SKIP_DQ, _native.KVAX_FA_SKIP_DKDV
+    SQ, SK = _native.KVAX_FA_SKIP_DQ, _native.KVAX_FA_SKIP_DKDV
 
     def fwd():
         flash_attention_forward(q, k, v, *ids, masks[0], w.scale, fp, bp, buffers=(out, lse))
@@ -181,27 +187,19 @@ def main():
             if events is not None:
                 events[i][1].record()
 
-    if args.pmc_calibration:
-        src = torch.ones(CALIBRATION_BYTES // 4, dtype=torch.float32, device=dev)
-        dst = torch.empty_like(src)
-        for _ in range(2):
-            torch.mul(src, 1.0, out=dst)  # elementwise kernel: reads and writes CALIBRATION_BYTES
-        torch.cuda.synchronize()
-        del src, dst
-
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    all_events = [[(ev(), ev()) for _ in phases] for _ in range(args.steps)]
+    all_events = [[(ev(), ev()) for _ in phases] for _ in range(steps)]
     t0 = time.perf_counter()
-    for s in range(args.steps):
-        step(all_events[s])
+    for s_ in range(steps):
+        step(all_events[s_])
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    kernel_ms = {name: float(np.mean([all_events[s][i][0].elapsed_time(all_events[s][i][1])
-                                      for s in range(args.steps)]))
-                 for i, (name, _) in enumerate(phases)}
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    kernel_ms = {name_: float(np.mean([all_events[s_][i][0].elapsed_time(all_events[s_][i][1])
+                                       for s_ in range(steps)]))
+                 for i, (name_, _) in enumerate(phases)}
 
     f_step = f_fwd * (3.5 if backward else 1.0)
     value = f_step / (ms_per_step * 1e-3) / 1e12
@@ -219,13 +217,49 @@ def main():
         gbps = alg_bytes / (kernel_ms["fa_fwd_kernel"] * 1e-3) / 1e9
         roofline = {"bound": "hbm", "kernel": "fa_fwd_kernel (split mode) + fa_fwd_combine_kernel",
                     "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
-                    "traffic": recorded_traffic("fa_fwd_kernel", args.workload),
+                    "traffic": recorded_traffic("fa_fwd_kernel", name),
                     "algorithmic_bytes": alg_bytes}
     else:
         roofline = {"bound": "mfma", "kernel": dominant, "achieved": achieved,
                     "peak": MFMA_BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
-                    "traffic": recorded_traffic(dominant, args.workload)}
+                    "traffic": recorded_traffic(dominant, name)}
+    figures = {
+        "value": value, "ms_per_step": ms_per_step, "pairs": pairs, "f_step": f_step, "f_fwd": f_fwd,
+        "roofline": roofline, "mask_build_ms": mask_ms, "kernel_ms": kernel_ms,
+        "kernel_tflops": {n: (kernel_flops[n] / (ms * 1e-3) / 1e12 if ms > 0 else 0.0)
+                          for n, ms in kernel_ms.items()},
+    }
+    return w, figures
+
+
+# The other configurations of the baseline, timed briefly after the headline one so that every
+# configuration has a figure in the same JSON line: (workload, mask block size)
+SECONDARY = [("dense_causal", 128), ("cp_shard", 128), ("block_skip", 128), ("block_skip", 64),
+             ("decode32k", 128)]
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); the path has no "
+              "collectives.  Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+
+    if args.pmc_calibration:
+        src = torch.ones(CALIBRATION_BYTES // 4, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            torch.mul(src, 1.0, out=dst)  # elementwise kernel: reads and writes CALIBRATION_BYTES
+        torch.cuda.synchronize()
+        del src, dst
+
+    w, m = measure(args, args.workload, args.block, args.steps, args.warmup)
+    backward = w.backward
     result = {
         # the headline metric's own wording for the configuration it is quoted on; `value` is its
         # forward+backward figure, the forward one and the mask build time follow as fwd_tflops and
@@ -235,12 +269,12 @@ def main():
                   ("doc-mask attention TFLOP/s, forward+backward, bf16, unmasked FLOPs" if backward
                    else "doc-mask attention TFLOP/s, forward, bf16, unmasked FLOPs"),
         "value_is": "forward+backward TFLOP/s" if backward else "forward TFLOP/s",
-        "value": value,
+        "value": m["value"],
         "unit": "TFLOP/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
+        "ms_per_step": m["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -251,21 +285,38 @@ def main():
             "seed": args.seed,
             "mask_block": args.block,
             "positions": "global" if args.global_positions else "restart per document",
-            "unmasked_pairs": pairs,
-            "flops_per_step": f_step,
+            "unmasked_pairs": m["pairs"],
+            "flops_per_step": m["f_step"],
             "num_documents": len(w.meta.get("doc_lengths", [])) or None,
             "padding_tokens": w.meta.get("pad"),
         },
-        "roofline": roofline,
-        "step_frac_of_mfma_peak": value / MFMA_BF16_DENSE_PEAK_TFLOPS,
-        "fwd_tflops": f_fwd / (kernel_ms["fa_fwd_kernel"] * 1e-3) / 1e12,
-        "mask_build_ms": mask_ms,
-        "kernel_ms": kernel_ms,
-        "kernel_tflops": {n: (kernel_flops[n] / (ms * 1e-3) / 1e12 if ms > 0 else 0.0)
-                          for n, ms in kernel_ms.items()},
+        "roofline": m["roofline"],
+        "step_frac_of_mfma_peak": m["value"] / MFMA_BF16_DENSE_PEAK_TFLOPS,
+        "fwd_tflops": m["f_fwd"] / (m["kernel_ms"]["fa_fwd_kernel"] * 1e-3) / 1e12,
+        "mask_build_ms": m["mask_build_ms"],
+        "kernel_ms": m["kernel_ms"],
+        "kernel_tflops": m["kernel_tflops"],
     }
+    if not args.no_secondary and args.workload == "doc32k":
+        others = {}
+        for name, block in SECONDARY:
+            torch.cuda.empty_cache()
+            w2, m2 = measure(args, name, block, args.secondary_steps, 3, device_tensors=True)
+            others[f"{name}@block{block}"] = {
+                "workload": WORKLOAD_TEXT[name], "mask_block": block, "steps": args.secondary_steps,
+                "value": m2["value"], "unit": "TFLOP/s",
+                "value_is": "forward+backward TFLOP/s" if w2.backward else "forward TFLOP/s",
+                "ms_per_step": m2["ms_per_step"], "unmasked_pairs": m2["pairs"],
+                "roofline": m2["roofline"], "mask_build_ms": m2["mask_build_ms"],
+                "kernel_ms": m2["kernel_ms"], "kernel_tflops": m2["kernel_tflops"],
+            }
+            del w2, m2
+        result["other_workloads"] = others
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(w, args.seed)
+        from kvax_amd.utils.benchmarking import workload
+        result["cpu_baseline"] = cpu_baseline(workload(args.workload, seed=args.seed,
+                                                       restart_positions=not args.global_positions,
+                                                       block=args.block), args.seed)
     print(json.dumps(result))
 
 

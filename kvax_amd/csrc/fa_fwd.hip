@@ -27,6 +27,8 @@ namespace {
 
 constexpr int kTK = kTileRows;  // kv rows per LDS tile
 
+constexpr float kRescaleStep = 8.f;  // log2 units
+
 struct FwdParams {
   const char* q;
   const char* k;
@@ -327,31 +329,37 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
           mx = fmaxf(mx, xor32(mx));
-          const float m_new = fmaxf(m_run[qt], mx * cs);
-          if (__any(m_new > m_run[qt])) {
+          // The running maximum only has to bound the scores loosely: it is raised (and O, l
+          // rescaled: 64 multiplies per lane) only when some row's maximum has grown by more than
+          // kRescaleStep, i.e. the exponentials below may reach 2^kRescaleStep instead of 1 - exact
+          // in the final O = acc / l and lse = m + log2(l), and no loss for a floating-point P.
+          // With a plain running maximum some of a wavefront's 32 rows raise it in most tiles.
+          if (__any(mx * cs > m_run[qt] + kRescaleStep)) {
+            const float m_new = fmaxf(m_run[qt], mx * cs);
             const float alpha = fast_exp2(m_run[qt] - m_new);
             l_run[qt] *= alpha;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
 #pragma unroll
               for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
+            m_run[qt] = m_new;
           }
-          m_run[qt] = m_new;
+          const float m_use = m_run[qt];
           float sum = 0.f;
 #pragma unroll
           for (int kt = 0; kt < 2; kt++) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-              const float e = fast_exp2(__builtin_fmaf(s[kt][qt][i], cs, -m_new));
-              s[kt][qt][i] = e;
-              sum += e;
-            }
+            for (int i = 0; i < 16; i++) s[kt][qt][i] = fast_exp2(__builtin_fmaf(s[kt][qt][i], cs, -m_use));
 #pragma unroll
-            for (int st = 0; st < 2; st++)
-              pb[kt][st][qt] = pack8<Tr>(s[kt][qt][8 * st + 0], s[kt][qt][8 * st + 1],
-                                         s[kt][qt][8 * st + 2], s[kt][qt][8 * st + 3],
-                                         s[kt][qt][8 * st + 4], s[kt][qt][8 * st + 5],
-                                         s[kt][qt][8 * st + 6], s[kt][qt][8 * st + 7]);
+            for (int st = 0; st < 2; st++) {
+              uint32_t w[4];
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                w[j] = Tr::pack2(s[kt][qt][8 * st + 2 * j], s[kt][qt][8 * st + 2 * j + 1]);
+                sum += s[kt][qt][8 * st + 2 * j] + s[kt][qt][8 * st + 2 * j + 1];
+              }
+              pb[kt][st][qt] = __builtin_bit_cast(vec8, make_uint4(w[0], w[1], w[2], w[3]));
+            }
           }
           l_run[qt] += sum;  // per half-wave partial; halves are added in the epilogue
         }

@@ -234,3 +234,30 @@ def test_too_long_key_sequences_are_refused_without_a_gpu():
     need = lib.kvax_fa_bwd_workspace_bytes(ctypes.byref(a))
     assert lib.kvax_fa_bwd(ctypes.byref(a), dummy, need, None) == -2
     assert b"LDS" in lib.kvax_last_error()
+
+
+def test_error_strings_are_per_thread():
+    """Two host threads fail in different ways at the same time, many times: each must read back its
+    own message (the last-error text is thread-local; no GPU is needed, nothing is launched)."""
+    import threading
+
+    lib = _native.lib()
+    problems = []
+
+    def worker(head_dim, expect):
+        a = _fa_args(1, 128, 128, 8, 2, head_dim)
+        for _ in range(2000):
+            rc = lib.kvax_fa_fwd(ctypes.byref(a), None, 0, None)
+            msg = lib.kvax_last_error()
+            if rc >= 0 or expect not in msg:
+                problems.append((head_dim, rc, msg))
+                return
+
+    # head_dim 100 is refused as unsupported; head_dim 128 with null tensors as a null pointer
+    threads = [threading.Thread(target=worker, args=(100, b"head_dim 100")),
+               threading.Thread(target=worker, args=(128, b"null tensor pointer"))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not problems, problems[:3]

@@ -344,3 +344,45 @@ def test_c_abi_rejects_bad_arguments_before_launching(device):
     assert lib.kvax_fa_bwd(C.byref(a), ws.data_ptr(), ws.numel(), stream) == -1
     assert b"gradient" in lib.kvax_last_error()
     assert good.abs().max() > 0
+
+
+def test_concurrent_host_threads(device):
+    """Two host threads call the forward at the same time, each on its own stream with its own
+    workspace and outputs (the library keeps no shared mutable state on this path; the kernels' LDS
+    limits are set under a once-flag).  Both must reproduce the single-threaded result bit for bit."""
+    import threading
+
+    from kvax_amd.ops.flash_attention import flash_attention_forward
+    from kvax_amd.utils.benchmarking import make_random_attention_inputs
+
+    params = FlashAttentionParamsConfig(128, 128)
+    cases = []
+    for i, (sq, hq, hkv, d) in enumerate([(2048, 8, 2, 128), (1536, 4, 4, 64)]):
+        data, scale = make_random_attention_inputs(2, sq, sq, hq, hkv, d, d, seed=40 + i, num_pad_tokens=100,
+                                                   device=device)
+        with attention_specs(*TP_SPECS):
+            masks = create_attention_mask(*data[3:], fwd_params=params)
+        want = flash_attention_forward(*data, masks[0], scale, params, params)
+        cases.append((data, scale, masks, want))
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def worker(i):
+        try:
+            data, scale, masks, _ = cases[i]
+            stream = torch.cuda.Stream(device=device)
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    results[i] = flash_attention_forward(*data, masks[0], scale, params, params)
+            stream.synchronize()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for (_, _, _, want), got in zip(cases, results):
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
