@@ -348,38 +348,64 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
 // work while the other has MFMAs.  The work-group streams the live Q / dO tiles of every query
 // head of the group; Q tiles stay one step longer than dO tiles, hence separate rings.
 // ---------------------------------------------------------------------------------------------
+// Shape of a dK/dV work-group per head_dim.  Up to 128 it is 8 wavefronts (4 role pairs, 128 kv
+// rows) at two per SIMD, stepping through 64-row query tiles.  At 256 a wavefront's fragments and
+// accumulators need more than half a SIMD's registers, so it is 4 wavefronts (2 pairs, 64 kv rows) at
+// one per SIMD, and the Q / dO rings only fit in LDS with 32-row steps: a 64-row tile of the live
+// list is then taken as two steps.
+template <int D>
+struct DkdvCfg {
+  static constexpr int kPairs = D > 128 ? 2 : 4;
+  static constexpr int kStepRows = D > 128 ? 32 : 64;  // query rows per step (and LDS stage)
+  static constexpr int kWps = D > 128 ? 1 : 2;         // wavefronts per SIMD
+  static constexpr int kWaves = 2 * kPairs;
+  static constexpr int kKvRows = 32 * kPairs;          // kv rows per work-group
+  static constexpr int kUnits = kStepRows / 32;        // 32-row MFMA units per step
+  static constexpr int kSub = kTile / kStepRows;       // steps per 64-row tile of the live list
+};
+
 template <int D>
 struct DkdvSmem {
-  static constexpr int kTileBytes = kTile * D * 2;  // swizzled, unpadded
-  static constexpr int kRowData = 4 * kTile * 4;    // lse, delta, seg, pos
+  using Cfg = DkdvCfg<D>;
+  static constexpr int kTileBytes = Cfg::kStepRows * D * 2;  // swizzled, unpadded
+  // lse, delta, seg, pos: 64 entries each whatever the step size (a wave-wide copy brings 64)
+  static constexpr int kRowData = 4 * kTile * 4;
   static constexpr int kQStages = 4, kDoStages = 3;
   static constexpr int kQ = 0;
   static constexpr int kDo = kQ + kQStages * kTileBytes;
   static constexpr int kRows = kDo + kDoStages * kTileBytes;
   static constexpr int kExchange = kRows + kQStages * kRowData;
-  // per pair two slots of P (one 64 x 32 tile, 16 bits per element): written for tile t while the
-  // slot of tile t - 1 is read
-  static constexpr int kTotal = kExchange + 4 * 2 * 4096;
+  // per pair two slots of P (one kStepRows x 32 tile, 16 bits per element): written for step s while
+  // the slot of step s - 1 is read
+  static constexpr int kSlotBytes = Cfg::kUnits * 2 * 1024;
+  static constexpr int kTotal = kExchange + Cfg::kPairs * 2 * kSlotBytes;
 };
 
-template <class Tr, int D, int WPS>
-__global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p) {
+template <class Tr, int D>
+__global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_bwd_dkdv_kernel(const BwdParams p) {
   using vec8 = typename Tr::vec8;
   using Smem = DkdvSmem<D>;
-  constexpr int NW = 8;
-  constexpr int TKV = 128;
+  using Cfg = DkdvCfg<D>;
+  constexpr int NW = Cfg::kWaves;
+  constexpr int NP = Cfg::kPairs;
+  constexpr int TKV = Cfg::kKvRows;
+  constexpr int SR = Cfg::kStepRows;
+  constexpr int UNITS = Cfg::kUnits;
+  constexpr int SUB = Cfg::kSub;
   constexpr int KSTEPS = D / 16;
   constexpr int DT = D / 32;
   constexpr int RB = D * 2;
-  // only the four P waves issue tile copies: they are the ones with slack before the barrier
-  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTile, D, 4>() + 1;
+  // only the P waves issue tile copies: they are the ones with slack before the barrier.  Each
+  // also copies its share of the four row-data arrays.
+  constexpr int kRowCopies = 4 / NP;
+  constexpr int kCopies = 2 * async_tile_copies_per_wave<SR, D, NP>() + kRowCopies;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;  // wave-uniform on purpose
   const int c = lane % 32, h = lane / 32;
-  const int pair = wave & 3;
-  const bool p_wave = wave < 4;  // role, wave-uniform
+  const int pair = wave % NP;
+  const bool p_wave = wave < NP;  // role, wave-uniform
 
   // kv tiles in the computed dispatch order (without one: early tiles first, which see the most
   // queries under a causal mask)
@@ -441,7 +467,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     compact_live_tiles<NW, true>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
   __syncthreads();
   const int n_live = *live_count;
-  const int steps = n_live * p.group;  // every head of the group walks the same list
+  const int steps = n_live * p.group * SUB;  // every head of the group walks the same list
 
   if (steps > 0) {
     // stationary fragments: K (negated when the scale is negative) for the P wave, V for the S wave
@@ -468,8 +494,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     }
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
-    const int which = pair;  // row-data array this P wave copies: lse, delta, seg, pos
-    const AsyncTileCopy<kTile, D, 4> copy_q(p.q_ss * 2, pair, lane), copy_do(p.do_ss * 2, pair, lane);
+    const AsyncTileCopy<SR, D, NP> copy_q(p.q_ss * 2, pair, lane), copy_do(p.do_ss * 2, pair, lane);
     // Step s = (head s / n_live of the group, list entry s % n_live); its Q tile and row data go to
     // slot s % 4 of their rings, its dO tile to slot s % 3.  The issuing side keeps its own cursor
     // (list index, per-head base pointers) and advances it by additions only: divisions and 64-bit
@@ -477,37 +502,50 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     const int head0 = kv_head * p.group;
     const char* is_q = p.q + ((int64_t)b * p.q_sb + (int64_t)head0 * p.q_sh) * 2;
     const char* is_do = p.dout + ((int64_t)b * p.do_sb + (int64_t)head0 * p.do_sh) * 2;
-    // row-data array this wave copies: lse, delta (per head) or seg, pos (per batch row)
-    const char* is_rows = which == 0   ? (const char*)(p.lse + ((int64_t)b * p.num_heads + head0) * p.q_len)
-                          : which == 1 ? (const char*)(p.delta + ((int64_t)b * p.num_heads + head0) * p.q_len)
-                          : which == 2 ? (const char*)(p.q_seg + (int64_t)b * p.q_len)
-                                       : (const char*)(p.q_pos + (int64_t)b * p.q_len);
-    const int64_t rows_per_head = which < 2 ? (int64_t)p.q_len * 4 : 0;
-    int is_li = 0;
+    // row-data arrays this wave copies (array w of lse, delta, seg, pos for w = pair, pair + NP, ...):
+    // lse and delta are per head, seg and pos per batch row
+    const char* is_rows[kRowCopies];
+    int64_t rows_per_head[kRowCopies];
+#pragma unroll
+    for (int r = 0; r < kRowCopies; r++) {
+      const int which = pair + r * NP;
+      is_rows[r] = which == 0   ? (const char*)(p.lse + ((int64_t)b * p.num_heads + head0) * p.q_len)
+                   : which == 1 ? (const char*)(p.delta + ((int64_t)b * p.num_heads + head0) * p.q_len)
+                   : which == 2 ? (const char*)(p.q_seg + (int64_t)b * p.q_len)
+                                : (const char*)(p.q_pos + (int64_t)b * p.q_len);
+      rows_per_head[r] = which < 2 ? (int64_t)p.q_len * 4 : 0;
+    }
+    int is_li = 0, is_sub = 0;
     uint32_t is_entry = live_list[0];
     auto issue_next = [&](int q_slot, int do_slot) {
-      const int qr0 = (int)(is_entry & 0xffffff) * kTile;
+      const int qr0 = (int)(is_entry & 0xffffff) * kTile + is_sub * SR;
       copy_q(is_q, qr0, p.q_len, smem_addr + Smem::kQ + q_slot * Smem::kTileBytes);
       copy_do(is_do, qr0, p.q_len, smem_addr + Smem::kDo + do_slot * Smem::kTileBytes);
-      async_copy_b32(is_rows + (int64_t)min(qr0 + lane, p.q_len - 1) * 4,
-                     __builtin_amdgcn_readfirstlane(smem_addr + Smem::kRows + q_slot * Smem::kRowData +
-                                                    which * (kTile * 4)));
-      if (++is_li == n_live) {
-        is_li = 0;
-        is_q += p.q_sh * 2;
-        is_do += p.do_sh * 2;
-        is_rows += rows_per_head;
+#pragma unroll
+      for (int r = 0; r < kRowCopies; r++)
+        async_copy_b32(is_rows[r] + (int64_t)min(qr0 + lane, p.q_len - 1) * 4,
+                       __builtin_amdgcn_readfirstlane(smem_addr + Smem::kRows + q_slot * Smem::kRowData +
+                                                      (pair + r * NP) * (kTile * 4)));
+      if (++is_sub == SUB) {
+        is_sub = 0;
+        if (++is_li == n_live) {
+          is_li = 0;
+          is_q += p.q_sh * 2;
+          is_do += p.do_sh * 2;
+#pragma unroll
+          for (int r = 0; r < kRowCopies; r++) is_rows[r] += rows_per_head[r];
+        }
+        is_entry = live_list[is_li];
       }
-      is_entry = live_list[is_li];
     };
 
     // P of the pair's tiles, 16-bit floats with a 10-bit mantissa whatever the tensor dtype:
     // [slot][unit mt][half st] x 64 lanes x 16 bytes, in the lane order of the C tile
-    char* exchange = smem + Smem::kExchange + pair * 8192 + lane * 16;
+    char* exchange = smem + Smem::kExchange + pair * 2 * Smem::kSlotBytes + lane * 16;
 
     // S wave, second part of a tile: dS = P * (dP - delta) rounded to the input dtype (masked
     // entries have P = 0), dK^T += Q^T dS.  x = dP of that tile.
-    auto finish_dk = [&](const f32x16 (&x)[2], const char* qtile, const float* delta_rows, const char* pslot) {
+    auto finish_dk = [&](const f32x16 (&x)[UNITS], const char* qtile, const float* delta_rows, const char* pslot) {
       vec8 ta[2][DT];
 #pragma unroll
       for (int st = 0; st < 2; st++)
@@ -515,7 +553,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
         for (int dt = 0; dt < DT; dt++)
           ta[st][dt] = tr_read_a_swz<Tr>(qtile + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
 #pragma unroll
-      for (int mt = 0; mt < 2; mt++) {
+      for (int mt = 0; mt < UNITS; mt++) {
         vec8 dsb[2];
 #pragma unroll
         for (int st = 0; st < 2; st++) {
@@ -533,18 +571,18 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
           dsb[st] = pack8<Tr>(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
         }
         vec8 tb[2][DT];  // operands of the next unit, requested before this unit's MFMAs
-        if (mt == 0) {
+        if (mt + 1 < UNITS) {
 #pragma unroll
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++)
-              tb[st][dt] = tr_read_a_swz<Tr>(qtile + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+              tb[st][dt] = tr_read_a_swz<Tr>(qtile + (32 * (mt + 1) + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
         }
 #pragma unroll
         for (int st = 0; st < 2; st++)
 #pragma unroll
           for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], dsb[st], acc[dt]);
-        if (mt == 0) {
+        if (mt + 1 < UNITS) {
 #pragma unroll
           for (int st = 0; st < 2; st++)
 #pragma unroll
@@ -553,7 +591,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
       }
     };
 
-    int li = 0;                    // list index of the current step
+    int li = 0, sub = 0;           // list index and sub-step of the current step
     uint32_t e0 = live_list[0];    // its entry
     uint32_t ep = 0;               // entry of the previous step
     if (p_wave) {
@@ -561,10 +599,10 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
       if (steps > 1) issue_next(1, 1);
     }
 
-    f32x16 x[2];  // S of this tile (P wave) / dP carried from the previous step (S wave)
+    f32x16 x[UNITS];  // S of this step (P wave) / dP carried from the previous step (S wave)
     int q_slot = 0, do_slot = 0, q_prev = 0;
     for (int step = 0; step < steps; step++) {
-      // the tile has landed; every wavefront is done with the previous step
+      // the rows of this step have landed; every wavefront is done with the previous step
       if (p_wave) {
         if (step + 1 < steps) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
       }
@@ -572,7 +610,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
       if (p_wave && step + 2 < steps) issue_next((q_slot + 2) & 3, do_slot >= 1 ? do_slot - 1 : 2);
       const int t = e0 & 0xffffff;
       const bool active = (e0 >> (24 + wave)) & 1, active_prev = (ep >> (24 + wave)) & 1;
-      const int qr0 = t * kTile;
+      const int qr0 = t * kTile + sub * SR;
       const char* qtile = smem + Smem::kQ + q_slot * Smem::kTileBytes;
       const char* dotile = smem + Smem::kDo + do_slot * Smem::kTileBytes;
       const float* rowdata = reinterpret_cast<const float*>(smem + Smem::kRows + q_slot * Smem::kRowData);
@@ -582,24 +620,24 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
       if (!p_wave && active_prev)
         finish_dk(x, smem + Smem::kQ + q_prev * Smem::kTileBytes,
                   reinterpret_cast<const float*>(smem + Smem::kRows + q_prev * Smem::kRowData) + kTile,
-                  exchange + ((step - 1) & 1) * 4096);
+                  exchange + ((step - 1) & 1) * Smem::kSlotBytes);
 
-      // 16 MFMAs per wavefront, S = Q K^T (P wave) or dP = dO V^T (S wave), both 32-row units
-      // interleaved; operand reads run four ahead of the MFMAs
+      // 8 * UNITS * KSTEPS / 8 MFMAs per wavefront, S = Q K^T (P wave) or dP = dO V^T (S wave), the
+      // 32-row units interleaved; operand reads run four ahead of the MFMAs
       const char* rows_a = p_wave ? qtile : dotile;
       if (active) {
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++)
+        for (int mt = 0; mt < UNITS; mt++)
 #pragma unroll
           for (int i = 0; i < 16; i++) x[mt][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++)
 #pragma unroll
-          for (int mt = 0; mt < 2; mt++)
+          for (int mt = 0; mt < UNITS; mt++)
             x[mt] = Tr::mfma(*reinterpret_cast<const vec8*>(rows_a + 32 * mt * RB + nat_off[ks]), frag[ks], x[mt]);
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-        for (int i = 0; i < 2 * KSTEPS - 4; i++) {
+        for (int i = 0; i < UNITS * KSTEPS - 4; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
@@ -614,10 +652,10 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
 #pragma unroll
           for (int dt = 0; dt < DT; dt++)
             ta[st][dt] = tr_read_a_swz<Tr>(dotile + 16 * st * RB, tr_off[dt][0], tr_off[dt][1]);
-        vec8 pb[2][2];
-        char* pslot = exchange + (step & 1) * 4096;
+        vec8 pb[UNITS][2];
+        char* pslot = exchange + (step & 1) * Smem::kSlotBytes;
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++) {
+        for (int mt = 0; mt < UNITS; mt++) {
           f32x16& sc = x[mt];
           if (!full)  // raw scores: masked -> -inf, so that P = exp2(-inf) = 0 (scale_log2_abs > 0)
             mask_c_tile<false>(sc, rowids, rowids + kTile, 32 * mt, qr0, h, kvseg, kvpos, col_lo,
@@ -641,20 +679,20 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
         }
         // dV^T += dO^T P
 #pragma unroll
-        for (int mt = 0; mt < 2; mt++) {
+        for (int mt = 0; mt < UNITS; mt++) {
           vec8 tb[2][DT];
-          if (mt == 0) {
+          if (mt + 1 < UNITS) {
 #pragma unroll
             for (int st = 0; st < 2; st++)
 #pragma unroll
               for (int dt = 0; dt < DT; dt++)
-                tb[st][dt] = tr_read_a_swz<Tr>(dotile + (32 + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+                tb[st][dt] = tr_read_a_swz<Tr>(dotile + (32 * (mt + 1) + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
           }
 #pragma unroll
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) acc[dt] = Tr::mfma(ta[st][dt], pb[mt][st], acc[dt]);
-          if (mt == 0) {
+          if (mt + 1 < UNITS) {
 #pragma unroll
             for (int st = 0; st < 2; st++)
 #pragma unroll
@@ -663,8 +701,11 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
         }
       }
       ep = e0;
-      li = li + 1 == n_live ? 0 : li + 1;
-      e0 = live_list[li];
+      if (++sub == SUB) {
+        sub = 0;
+        li = li + 1 == n_live ? 0 : li + 1;
+        e0 = live_list[li];
+      }
       q_prev = q_slot;
       q_slot = (q_slot + 1) & 3;
       do_slot = do_slot == 2 ? 0 : do_slot + 1;
@@ -674,7 +715,7 @@ __global__ __launch_bounds__(512, WPS) void fa_bwd_dkdv_kernel(const BwdParams p
     if (!p_wave && ((ep >> (24 + wave)) & 1))
       finish_dk(x, smem + Smem::kQ + q_prev * Smem::kTileBytes,
                 reinterpret_cast<const float*>(smem + Smem::kRows + q_prev * Smem::kRowData) + kTile,
-                exchange + ((steps - 1) & 1) * 4096);
+                exchange + ((steps - 1) & 1) * Smem::kSlotBytes);
   }
   __syncthreads();  // the next chunk reuses the bookkeeping, the rings and the exchange slots
   }
@@ -720,12 +761,12 @@ int reserve_lds(K kernel, int need, int bytes, LdsReservation* reservation, cons
   return reservation->ensure(kernel, bytes, what);
 }
 
-// dQ launch: NW wavefronts (32 query rows each) per work-group, two per SIMD.
-template <class Tr, int D, int NW, int STAGES>
+// dQ launch: NW wavefronts (32 query rows each) per work-group, WPS per SIMD.
+template <class Tr, int D, int NW, int STAGES, int WPS = 2>
 int launch_dq(BwdParams p, hipStream_t stream) {
-  auto kernel = fa_bwd_dq_kernel<Tr, D, NW, 2, STAGES>;
+  auto kernel = fa_bwd_dq_kernel<Tr, D, NW, WPS, STAGES>;
   static LdsReservation done;
-  constexpr int kLimit = kLdsPerCu / (8 / NW);
+  constexpr int kLimit = kLdsPerCu / (4 * WPS / NW);  // work-groups per compute unit share the LDS
   const int smem = DqSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   if (int rc = reserve_lds(kernel, smem, kLimit, &done, "the dQ kernel")) return rc;
   p.num_tiles = cdiv(p.q_len, NW * 32);
@@ -739,7 +780,8 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   // a key sequence too long for the dQ kernel's largest configuration is refused before anything
   // is enqueued (the dK/dV kernel has no such limit)
   if (p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ)) {
-    const int need = DqSmem<D, 3>::kTotal + live_tiles_bytes(8, p.n_kv_tiles);
+    const int need = D > 128 ? DqSmem<D, 2>::kTotal + live_tiles_bytes(4, p.n_kv_tiles)
+                             : DqSmem<D, 3>::kTotal + live_tiles_bytes(8, p.n_kv_tiles);
     if (need > kLdsPerCu)
       return fail(KVAX_EUNSUPPORTED, "the dQ kernel needs %d bytes of LDS for tile bitmaps (limit %d): "
                   "sequence too long", need, kLdsPerCu);
@@ -748,12 +790,14 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   {
     TileSummaryJob jobs[2] = {{p.kv_pos, p.kv_seg, (void*)p.kv_tiles, p.kv_len},
                               {p.q_pos, p.q_seg, (void*)p.q_tiles, p.q_len}};
-    int32_t* counters = tile_order_counters(p.order_ws, p.batch, cdiv(p.kv_len, 128));
+    int32_t* counters = tile_order_counters(p.order_ws, p.batch, cdiv(p.kv_len, DkdvCfg<D>::kKvRows));
     if (int rc = launch_tile_summaries(jobs, 2, p.batch, stream, counters)) return rc;
   }
   // dQ: two work-groups of four wavefronts per compute unit (each hides the other's prologue,
-  // barriers and final stores) when the tile bitmaps fit beside the smaller ring, else one of eight
-  constexpr int kStagesSmall = D == 128 ? 2 : 3;
+  // barriers and final stores) when the tile bitmaps fit beside the smaller ring, else one of eight;
+  // at head_dim 256 (128 accumulator registers for dQ alone) one work-group of four, one per SIMD
+  constexpr int kStagesSmall = D == 64 ? 3 : 2;
+  using Cfg = DkdvCfg<D>;
   const bool run_dq = p.q_len > 0 && !(p.flags & KVAX_FA_SKIP_DQ);
   const bool run_dkdv = p.kv_len > 0 && !(p.flags & KVAX_FA_SKIP_DKDV);
   const bool dq_small =
@@ -761,26 +805,30 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
   // dK/dV runs one long work-group per compute unit: its light work items are dispatched last, by
   // decreasing number of live tiles, so that the launch does not end on a few long ones
   {
-    const int items = cdiv(p.kv_len, 128);
+    const int items = cdiv(p.kv_len, Cfg::kKvRows);
     if (run_dkdv && items >= kMinOrderedItems && items <= kMaxOrderedItems &&
         (int64_t)items * (p.n_q_tiles + 2) < 0x7fffffff) {
       const TileOrderJob job{p.kv_tiles, p.q_tiles, p.order_ws, p.n_kv_tiles, p.n_q_tiles,
-                             128 / kTileRows, items, 0};
+                             Cfg::kKvRows / kTileRows, items, 0};
       if (int rc = launch_tile_order(job, p.batch, stream)) return rc;
       p.dkdv_order = p.order_ws;
     }
   }
   if (run_dq) {
-    if (dq_small) {
-      if (int rc = launch_dq<Tr, D, 4, kStagesSmall>(p, stream)) return rc;
+    if constexpr (D > 128) {
+      if (int rc = launch_dq<Tr, D, 4, 2, 1>(p, stream)) return rc;
     } else {
-      if (int rc = launch_dq<Tr, D, 8, 3>(p, stream)) return rc;
+      if (dq_small) {
+        if (int rc = launch_dq<Tr, D, 4, kStagesSmall>(p, stream)) return rc;
+      } else {
+        if (int rc = launch_dq<Tr, D, 8, 3>(p, stream)) return rc;
+      }
     }
   }
-  // dK/dV: 8 wavefronts in 4 role pairs (128 kv rows) per work-group, two per SIMD
+  // dK/dV: wavefronts in role pairs (see DkdvCfg)
   if (run_dkdv) {
-    constexpr int NW = 8;
-    auto kernel = fa_bwd_dkdv_kernel<Tr, D, 2>;
+    constexpr int NW = Cfg::kWaves;
+    auto kernel = fa_bwd_dkdv_kernel<Tr, D>;
     static LdsReservation done;
     // live-tile bookkeeping for as many query tiles as the remaining LDS holds (a multiple of 64)
     constexpr int kLdsLimit = kLdsPerCu;
@@ -789,7 +837,7 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     p.list_tiles = min(chunk, max(p.n_q_tiles, 1));
     const int smem = DkdvSmem<D>::kTotal + live_tiles_bytes(NW, p.list_tiles);
     if (int rc = reserve_lds(kernel, smem, kLdsLimit, &done, "the dK/dV kernel")) return rc;
-    p.num_tiles = cdiv(p.kv_len, 128);
+    p.num_tiles = cdiv(p.kv_len, Cfg::kKvRows);
     p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, 1}.grid();
     hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dkdv_kernel")) return rc;
@@ -811,7 +859,7 @@ extern "C" size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* a) {
   // delta [batch, heads, q_len] fp32, the tile summaries of the kv and query sequences, and the
   // dispatch order of the dK/dV work items
   return delta_bytes(a) + tile_summary_bytes(a->batch, a->kv_len) + tile_summary_bytes(a->batch, a->q_len) +
-         tile_order_bytes(a->batch, cdiv(a->kv_len, 128));
+         tile_order_bytes(a->batch, cdiv(a->kv_len, a->head_dim > 128 ? 64 : 128));
 }
 
 extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t workspace_bytes,
@@ -877,6 +925,8 @@ extern "C" int kvax_fa_bwd(const kvax_fa_args* a, void* workspace, size_t worksp
   p.k_sign = a->scale < 0.f ? 0x80008000u : 0u;
   hipStream_t stream = (hipStream_t)stream_;
   const bool bf16 = a->dtype == KVAX_BF16;
+  if (a->head_dim == 256)
+    return bf16 ? launch_bwd<Bf16, 256>(p, stream) : launch_bwd<F16, 256>(p, stream);
   if (a->head_dim == 128)
     return bf16 ? launch_bwd<Bf16, 128>(p, stream) : launch_bwd<F16, 128>(p, stream);
   return bf16 ? launch_bwd<Bf16, 64>(p, stream) : launch_bwd<F16, 64>(p, stream);

@@ -266,7 +266,10 @@ __device__ __forceinline__ void mask_c_tile(f32x16& s, const int32_t* row_seg, c
 // ---------------------------------------------------------------------------------------------
 template <int D>
 __device__ __forceinline__ int swz(int r) {
-  if (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);
+  // D == 128, 256: rows are one or two full turns of the 64 banks apart, so the chunk position
+  // modulo 16 decides the banks and one 4-bit pattern serves both (at 256 it permutes the chunks
+  // within each half of the row)
+  if (D >= 128) return ((r & 3) << 2) | ((r >> 2) & 3);
   return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);  // D == 64: 8 chunks per row
 }
 

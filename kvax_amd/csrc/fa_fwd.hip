@@ -479,8 +479,9 @@ FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv
   if (batch <= 0 || q_len <= 0 || kv_len <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return plan;
   const int n_kv_tiles = cdiv(kv_len, kTileRows);
   const int64_t regular = (int64_t)batch * num_heads * cdiv(q_len, kSplitTileRows);
-  const int ring_bytes = (2 * kTK * head_dim * 2 + 2 * kTK * 4) * (head_dim == 128 ? 2 : 3);
-  if (ring_bytes + live_tiles_bytes(4, n_kv_tiles) > kLdsHalfCu) return plan;
+  // the ring of the four-wavefront configuration (see launch_fwd_auto) and its share of the LDS
+  const int ring_bytes = (2 * kTK * head_dim * 2 + 2 * kTK * 4) * (head_dim == 64 ? 3 : 2);
+  if (ring_bytes + live_tiles_bytes(4, n_kv_tiles) > (head_dim == 256 ? kLdsPerCu : kLdsHalfCu)) return plan;
   if (q_len >= kSplitTileRows && regular >= 256) return plan;
   plan.split_mode = true;
   const int64_t rows = (int64_t)q_len * (num_heads / num_kv_heads);
@@ -538,11 +539,18 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
 // otherwise one work-group of eight wavefronts.
 template <class Tr, int D>
 int launch_fwd_auto(const FwdParams& p, hipStream_t stream) {
-  constexpr int kStagesSmall = D == 128 ? 2 : 3;
-  if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall, true>(p, stream);
-  const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
-  if (small <= kLdsHalfCu) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
-  return launch_fwd<Tr, D, 1, 8, 2, 3>(p, stream);
+  if constexpr (D == 256) {
+    // 128 accumulator registers for O and 64 for the Q fragments: one wavefront per SIMD, one
+    // work-group of four per compute unit, two 64.5 KB stages
+    if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 1, 2, true>(p, stream);
+    return launch_fwd<Tr, D, 1, 4, 1, 2>(p, stream);
+  } else {
+    constexpr int kStagesSmall = D == 128 ? 2 : 3;
+    if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall, true>(p, stream);
+    const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
+    if (small <= kLdsHalfCu) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
+    return launch_fwd<Tr, D, 1, 8, 2, 3>(p, stream);
+  }
 }
 
 }  // namespace
@@ -554,8 +562,8 @@ int validate_fa_common(const kvax_fa_args* a) {
   if (a->num_heads % a->num_kv_heads)
     return fail(KVAX_EINVAL, "num_heads %d is not a multiple of num_kv_heads %d", a->num_heads,
                 a->num_kv_heads);
-  if (a->head_dim != 64 && a->head_dim != 128)
-    return fail(KVAX_EUNSUPPORTED, "head_dim %d is not built (64 and 128 are)", a->head_dim);
+  if (a->head_dim != 64 && a->head_dim != 128 && a->head_dim != 256)
+    return fail(KVAX_EUNSUPPORTED, "head_dim %d is not built (64, 128 and 256 are)", a->head_dim);
   if (a->dtype != KVAX_BF16 && a->dtype != KVAX_F16)
     return fail(KVAX_EUNSUPPORTED, "dtype %d is not supported (bf16 and f16 are)", a->dtype);
   if (a->flags & ~(KVAX_FA_DKDV_F32 | KVAX_FA_SKIP_DELTA | KVAX_FA_SKIP_DQ | KVAX_FA_SKIP_DKDV)) return fail(KVAX_EINVAL, "unknown bits in flags");
@@ -691,8 +699,8 @@ int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, 
   hipStream_t stream = (hipStream_t)stream_;
   if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
   {  // too long for the largest configuration: refuse before anything is enqueued
-    const int ring = (2 * kTK * a->head_dim * 2 + 2 * kTK * 4) * 3;
-    const int need = ring + live_tiles_bytes(8, p.n_kv_tiles);
+    const int ring = (2 * kTK * a->head_dim * 2 + 2 * kTK * 4) * (a->head_dim == 256 ? 2 : 3);
+    const int need = ring + live_tiles_bytes(a->head_dim == 256 ? 4 : 8, p.n_kv_tiles);
     if (need > kLdsPerCu)
       return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
                   a->kv_len, need, kLdsPerCu);
@@ -702,6 +710,8 @@ int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, 
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
   const bool bf16 = a->dtype == KVAX_BF16;
+  if (a->head_dim == 256)
+    return bf16 ? launch_fwd_auto<Bf16, 256>(p, stream) : launch_fwd_auto<F16, 256>(p, stream);
   if (a->head_dim == 128)
     return bf16 ? launch_fwd_auto<Bf16, 128>(p, stream) : launch_fwd_auto<F16, 128>(p, stream);
   return bf16 ? launch_fwd_auto<Bf16, 64>(p, stream) : launch_fwd_auto<F16, 64>(p, stream);

@@ -29,10 +29,10 @@ from kvax_amd.utils.sharding import context_parallel_degree
 from kvax_amd.utils.specs import get_attention_specs
 from kvax_amd.utils.typing import AttentionMask, DeviceArray
 
-SUPPORTED_HEAD_DIMS = (64, 128)  # what the kernels are built for
-# What ``flash_attention`` takes for query/key (the reference's list, flash_attention_triton.py:1397,
-# up to the largest built size); smaller ones and a different value head_dim are zero-padded.
-ACCEPTED_HEAD_DIMS = (16, 32, 64, 128)
+SUPPORTED_HEAD_DIMS = (64, 128, 256)  # what the kernels are built for
+# What ``flash_attention`` takes for query/key: the reference's list (flash_attention_triton.py:1397).
+# Sizes between the built ones (16, 32, 192) and a different value head_dim are zero-padded.
+ACCEPTED_HEAD_DIMS = (16, 32, 64, 128, 192, 256)
 _DTYPES = {torch.bfloat16: _native.KVAX_BF16, torch.float16: _native.KVAX_F16}
 
 
@@ -277,8 +277,8 @@ def flash_attention(
     ``[lower_full, upper_full)`` is computed from per-block id extremes and is only right for such
     layouts; the kernels trust it, so ids that return to an earlier value give wrong results
     without an error.  Ids need not be sorted or dense (``5 5 2 2 7`` is fine).
-    Query/key head dims 16, 32, 64, 128 and any value head dim up to 128 are taken (the kernels run
-    at 64 or 128; other sizes are zero-padded here).
+    Query/key head dims 16, 32, 64, 128, 192, 256 and any value head dim up to 256 are taken (the
+    kernels run at 64, 128 or 256; other sizes are zero-padded here).
     ``memory_optimized_gqa_backward`` is accepted and has no effect: dK/dV are always reduced
     over the query heads of a group inside the kernel, which is what the flag asks for.
     ``debug`` is accepted and ignored.  With ``assume_sequential_positions`` the causal test uses

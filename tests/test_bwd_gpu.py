@@ -114,6 +114,45 @@ def test_backward_small_and_unequal_head_dims(device, d_qk, d_v, hq, hkv):
     check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if hkv == 1 else ATOL)
 
 
+# head_dim 256: four wavefronts per dK/dV work-group (64 kv rows), 32-row query steps; 192 is padded
+@pytest.mark.parametrize("sq, sk, hq, hkv, d, pad, nseg, fwd_blocks, bwd_blocks", [
+    (384, 384, 4, 4, 256, 0, 1, (64, 64), (64, 64)),
+    (256, 256, 8, 2, 256, 100, 1, (128, 128), (64, 128)),
+    (1024, 1024, 8, 2, 256, 77, 5, (128, 128), (128, 128)),
+    (2048, 2048, 4, 4, 256, 300, 7, (64, 64), (128, 64)),
+    (512, 1024, 4, 2, 256, 0, 1, (128, 128), (128, 128)),
+    (1024, 1024, 4, 1, 192, 50, 12, (64, 64), (64, 64)),
+    (2304, 2304, 2, 2, 256, 0, 3, (128, 128), (128, 128)),   # more kv work items than the ordering threshold
+])
+def test_backward_large_head_dims(device, sq, sk, hq, hkv, d, pad, nseg, fwd_blocks, bwd_blocks):
+    lengths = generate_random_segments_lengths(min(sq, sk), nseg)
+    start = sk - sq if sk > sq else 0
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d, d, seed=sq + d + hq,
+                                               num_pad_tokens=pad, start_query_position=start,
+                                               list_of_segment_lengths=lengths, device=device)
+    dout = torch.randn(data[0].shape, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(device)
+    out, dq, dk, dv = run_backward(data, scale, fwd_blocks, bwd_blocks, dout)
+    q_, k_, v_, *ids_ = [x.cpu() for x in data]
+    ref_out, _ = ao.attention_forward(q_.float().numpy(), k_.float().numpy(), v_.float().numpy(),
+                                      *[x.numpy() for x in ids_], scale)
+    check_grad("out", out, ref_out)
+    check_all((dq, dk, dv), oracle_backward(data, scale, dout), data[4], data[6])
+
+
+def test_backward_head_dim_256_positions_restart(device):
+    """The over-covering masks (positions restart per document) at head_dim 256, both block sizes."""
+    w = workload("cpu_plumbing")
+    g = torch.Generator().manual_seed(5)
+    shape_q, shape_k = (1, w.q_len, 8, 256), (1, w.kv_len, 2, 256)
+    q, k, v, dout = (torch.randn(sh, generator=g).to(torch.bfloat16).to(device)
+                     for sh in (shape_q, shape_k, shape_k, shape_q))
+    data = (q, k, v) + w.ids(device)
+    scale = 256 ** -0.5
+    for blocks in ((64, 64), (128, 128)):
+        _, dq, dk, dv = run_backward(data, scale, blocks, blocks, dout)
+        check_all((dq, dk, dv), oracle_backward(data, scale, dout), data[4], data[6])
+
+
 @pytest.mark.parametrize("case", [CASES[7], CASES[6], CASES[8]])
 def test_fp32_dkdv_within_plain_bound(device, case):
     """dK/dV straight from the fp32 accumulators: plain max abs error <= 2e-2, no relative term."""

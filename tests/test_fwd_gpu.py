@@ -102,14 +102,38 @@ def test_forward_small_and_unequal_head_dims(device, sq, sk, hq, hkv, d_qk, d_v,
     check(out, oracle_forward(data, scale), data[4])
 
 
+# head_dim 256 runs natively (one wavefront per SIMD), 192 through zero padding to 256; the list of
+# sizes is the reference's (flash_attention_triton.py:1397-1403)
+@pytest.mark.parametrize("sq, sk, hq, hkv, d_qk, d_v, pad, nseg, block", [
+    (384, 384, 4, 4, 256, 256, 0, 1, 64),
+    (400, 300, 4, 2, 256, 256, 0, 1, 128),
+    (1024, 1024, 8, 2, 256, 256, 77, 5, 128),
+    (2048, 2048, 4, 1, 256, 256, 300, 7, 64),
+    (512, 512, 4, 2, 192, 192, 50, 3, 64),
+    (384, 384, 4, 4, 192, 128, 0, 1, 64),
+    (384, 384, 4, 4, 128, 256, 30, 2, 64),
+    (1, 4096, 16, 4, 256, 256, 0, 1, 128),      # decode: split mode at head_dim 256
+    (8, 3000, 8, 2, 192, 192, 0, 1, 128),
+])
+def test_forward_large_head_dims(device, sq, sk, hq, hkv, d_qk, d_v, pad, nseg, block):
+    lengths = generate_random_segments_lengths(min(sq, sk), nseg) if sq > 8 else None
+    start = sk - sq if sq <= 8 else 0
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d_qk, d_v, seed=sq + sk + d_qk,
+                                               num_pad_tokens=pad, start_query_position=start,
+                                               list_of_segment_lengths=lengths, device=device)
+    out = run_forward(data, scale, block, block)
+    assert out.shape == (2, sq, hq, d_v)
+    check(out, oracle_forward(data, scale), data[4])
+
+
 def test_head_dims_that_are_not_taken(device):
-    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 256, 256, device=device)
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 512, 512, device=device)
     with pytest.raises(ValueError, match="hid_dim"):
         run_forward(data, scale, 64, 64)
     data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 24, 24, device=device)
     with pytest.raises(ValueError, match="hid_dim"):
         run_forward(data, scale, 64, 64)
-    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 64, 192, device=device)
+    data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 64, 320, device=device)
     with pytest.raises(ValueError, match="value head_dim"):
         run_forward(data, scale, 64, 64)
 

@@ -331,7 +331,7 @@ def test_c_abi_rejects_bad_arguments_before_launching(device):
     assert fwd(a) == -2 and b"stride" in lib.kvax_last_error()
     a = args(); a.dtype = 5
     assert fwd(a) == -2
-    a = args(); a.head_dim = 256
+    a = args(); a.head_dim = 96
     assert fwd(a) == -2 and b"head_dim" in lib.kvax_last_error()
     a = args(); a.fwd_query_block = 0
     assert fwd(a) == -1
