@@ -24,7 +24,7 @@ typedef void* kvax_stream_t; /* a hipStream_t (NULL = the null stream) */
 enum {
   KVAX_OK = 0,
   KVAX_EINVAL = -1,       /* bad shape / flag / null pointer */
-  KVAX_EUNSUPPORTED = -2, /* valid request that the kernels do not cover (e.g. head_dim) */
+  KVAX_EUNSUPPORTED = -2, /* valid request that the kernels do not cover (e.g. head_dim 96) */
   KVAX_EWORKSPACE = -3,   /* workspace missing or too small */
   KVAX_ELAUNCH = -4       /* HIP reported a launch error */
 };
@@ -79,7 +79,8 @@ int kvax_mask_build(const int32_t* q_pos, const int32_t* q_seg, const int32_t* k
  * query heads of a group (:1855-1868).
  *
  * Tensors are consumed in the public [batch, seq, heads, head_dim] layout through element
- * strides {batch, seq, head}; the head_dim axis must be contiguous.  Sequence lengths need not
+ * strides {batch, seq, head}; the head_dim axis must be contiguous and head_dim is 64, 128 or 256
+ * (the reference's other sizes, :1397-1403, are zero-padded to these by the caller).  Sequence lengths need not
  * be multiples of the block sizes: tails are handled inside the kernels.  The reference's
  * assume_sequential_positions mode (causal test on token indices plus a per-shard offset,
  * :1421-1451) needs no kernel support: the caller passes those indices as q_pos / kv_pos.
