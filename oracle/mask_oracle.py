@@ -19,9 +19,12 @@ Three independent statements of the same function, used to pin each other:
 Parity status: pinned by (1) agreement loop == summaries on random inputs, (2) agreement with
 the dense definition on the reference test's own input family (regenerated exactly: its
 segment lengths come from Python's ``random.seed(0)``, kvax/utils/benchmarking.py:309-324),
-(3) closed forms for a single causal document, (4) invariants.  In the regime where the
-heuristic departs from any/all the step-by-step restatement is the only authority (the
-reference holds no stored vectors and cannot run here).
+(3) closed forms for a single causal document, (4) invariants, (5) in the regime where the
+heuristic departs from any/all (positions restarting per document, unsorted ids, padding in the
+middle, ragged lengths) vectors worked out by hand from the reference's kernel and host glue,
+block by block, with the derivation written next to them (tests/golden/mask_hand_worked.json):
+the reference holds no stored vectors and cannot run here, so those are the independent check
+that a misread index, comparison or sentinel rule would fail.
 """
 from __future__ import annotations
 
