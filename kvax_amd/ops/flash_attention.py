@@ -281,11 +281,12 @@ def flash_attention(
     kernels run at 64, 128 or 256; other sizes are zero-padded here).
     ``memory_optimized_gqa_backward`` is accepted and has no effect: dK/dV are always reduced
     over the query heads of a group inside the kernel, which is what the flag asks for.
-    ``debug`` is accepted and ignored.  With ``assume_sequential_positions`` the causal test uses
+    ``debug`` (passed to the Triton launcher in the reference) checks the precondition below on the
+    ids and raises ``ValueError`` when it does not hold.  With ``assume_sequential_positions`` the causal test uses
     token indices (plus the shard offset under context parallelism, :1421-1451) instead of the
     position arrays; the indices are materialised here and passed as positions.
     """
-    del memory_optimized_gqa_backward, debug
+    del memory_optimized_gqa_backward
     if bias is not None:
         raise NotImplementedError("Bias is not supported in Flash multi head attention")
     if mask is None or len(mask) == 0:
@@ -294,6 +295,9 @@ def flash_attention(
         raise ValueError(f"The case with num_mask_tensors={len(mask)} is not supported.")
     get_attention_specs()
     _check_inputs(query, key, value)
+    if debug:
+        _check_documents_are_contiguous(query_segment_ids, "query_segment_ids")
+        _check_documents_are_contiguous(kv_segment_ids, "kv_segment_ids")
     cp = context_parallel_degree(mesh)
     if fwd_params is None:
         fwd_params = get_default_flash_attention_params(backward=False)
@@ -319,6 +323,21 @@ def flash_attention(
         query, key, value, query_positions, query_segment_ids, kv_positions, kv_segment_ids,
         tuple(mask), float(scale), fwd_params, bwd_params, cp)
     return out if d_v == d_run else out[..., :d_v]
+
+
+def _check_documents_are_contiguous(segment_ids: torch.Tensor, name: str) -> None:
+    """Raises ValueError when, along some row, a segment id comes back after another id has followed
+    it (padding, id -1, is ignored): the number of runs of equal ids must equal the number of ids."""
+    for b in range(segment_ids.shape[0]):
+        row = segment_ids[b]
+        row = row[row != -1]
+        if row.numel() == 0:
+            continue
+        runs = 1 + int((row[1:] != row[:-1]).sum().item())
+        if runs != torch.unique(row).numel():
+            raise ValueError(
+                f"{name}[{b}]: a segment id comes back after another one has followed it; the block "
+                "mask and the attention kernels need every document to be one contiguous run")
 
 
 def _sequential_positions(query, key, cp: int, permuted: bool):

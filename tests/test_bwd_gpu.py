@@ -328,10 +328,12 @@ def test_missing_backward_masks(device):
             out.sum().backward()
 
 
-def _random_case(seed):
+def _random_case(seed, head_dim=None):
     """Seeded random shapes, documents, padding, block sizes and head layouts."""
     rng = np.random.default_rng(seed)
     d = int(rng.choice([64, 128]))
+    if head_dim is not None:
+        d = head_dim
     hkv = int(rng.choice([1, 2, 4]))
     hq = hkv * int(rng.choice([1, 2, 4, 8]))
     block = int(rng.choice([64, 128]))
@@ -347,9 +349,11 @@ def _random_case(seed):
                 restart=bool(rng.random() < 0.5))
 
 
-@pytest.mark.parametrize("seed", range(16))
-def test_randomized_shapes_forward_and_backward(device, seed):
-    c = _random_case(seed)
+# seeds 0-15 draw head_dim 64 or 128; the next eight repeat the draw at head_dim 256 (four wavefronts
+# per dK/dV work-group, two steps per 64-row query tile, GQA groups up to 8)
+@pytest.mark.parametrize("seed, head_dim", [(i, None) for i in range(16)] + [(100 + i, 256) for i in range(8)])
+def test_randomized_shapes_forward_and_backward(device, seed, head_dim):
+    c = _random_case(seed, head_dim)
     data, scale = make_random_attention_inputs(c["batch"], c["sq"], c["sk"], c["hq"], c["hkv"], c["d"], c["d"],
                                                seed=seed, num_pad_tokens=c["pad"],
                                                list_of_segment_lengths=c["lengths"], device=device)

@@ -239,6 +239,23 @@ def test_unsorted_document_ids(device):
         check(out, oracle_forward(data, scale), q_seg)
 
 
+def test_debug_flag_checks_the_document_layout(device):
+    """``debug=True`` verifies that no segment id returns after another one has followed it."""
+    data, scale = make_random_attention_inputs(1, 256, 256, 2, 2, 64, 64, num_pad_tokens=20,
+                                               list_of_segment_lengths=[100, 60, -1], device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(q_pos, q_seg, kv_pos, kv_seg)
+        flash_attention(q, k, v, q_pos, q_seg, kv_pos, kv_seg, mask, scale=scale, debug=True)  # fine
+        bad = kv_seg.clone()
+        bad[:, 200:210] = 0  # document 0 comes back inside document 2
+        with pytest.raises(ValueError, match="comes back"):
+            flash_attention(q, k, v, q_pos, q_seg, kv_pos, bad, mask, scale=scale, debug=True)
+        ok = kv_seg.clone()
+        ok[:, 120:125] = -1  # padding in the middle of a document does not split it
+        flash_attention(q, k, v, q_pos, q_seg, kv_pos, ok, mask, scale=scale, debug=True)
+
+
 def test_errors(device):
     data, scale = make_random_attention_inputs(1, 128, 128, 2, 2, 64, 64, device=device)
     q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
