@@ -59,9 +59,10 @@ struct FwdParams {
   // pairs; work-group `split` of an item takes the kv tiles [split, split + 1) * split_tiles of the
   // item's range and leaves a partial result
   int num_splits, split_tiles;
+  int num_parts;              // partial results per item: num_splits, or twice that in narrow mode
   int part_rows;              // rows per tile that have a partial (<= TQ)
-  float* part_o;              // [items, num_splits, part_rows, D] unnormalised O
-  float* part_ml;             // [items, num_splits, part_rows, 2] running max (base 2) and sum
+  float* part_o;              // [items, num_parts, part_rows, D] unnormalised O
+  float* part_ml;             // [items, num_parts, part_rows, 2] running max (base 2) and sum
 };
 
 template <int D, int STAGES>
@@ -82,7 +83,9 @@ struct FwdSmem {
 // split_tiles tiles, one work-group each (those beyond the end of the range have nothing to do), each
 // leaving an unnormalised partial result that fa_fwd_combine_kernel merges.  Windows of one size
 // for all rows of the batch keep the work-groups equally long when the rows are not.
-template <class Tr, int D, int MQ, int NW, int WPS, int STAGES, bool SPLIT>
+// NARROW: split mode with at most 32 rows (decoding), where the four wavefronts share the arithmetic
+// of every tile instead of the rows (see the constants below).
+template <class Tr, int D, int MQ, int NW, int WPS, int STAGES, bool SPLIT, bool NARROW>
 __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p) {
   using vec8 = typename Tr::vec8;
   using Smem = FwdSmem<D, STAGES>;
@@ -91,12 +94,20 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   constexpr int DT = D / 32;      // 32-row tiles of O^T
   constexpr int RB = D * 2;       // bytes per tile row
   constexpr int kCopies = 2 * async_tile_copies_per_wave<kTK, D, NW>() + 1;  // per wave and tile
-  static_assert(STAGES == 2 || STAGES == 3, "the loop below keeps STAGES - 1 tiles in flight");
+  static_assert(STAGES >= 2 && STAGES <= 4, "the loop below keeps STAGES - 1 tiles in flight");
+  // NARROW (split mode with at most 32 rows, i.e. decoding): every wavefront takes the same rows and
+  // a quarter of the arithmetic of a tile - wavefront w the key rows [32 (w & 1), +32) and, of
+  // O^T += V^T P^T, the head-dim slices of half w >> 1 - instead of one wavefront working while three
+  // wait.  The two key halves keep separate running maxima and leave separate partial results.
+  static_assert(!NARROW || (SPLIT && NW == 4 && MQ == 1 && DT % 2 == 0), "narrow mode splits a tile four ways");
+  constexpr int KT = NARROW ? 1 : 2;         // 32-key halves of a tile per wavefront
+  constexpr int DTO = NARROW ? DT / 2 : DT;  // 32-row slices of O^T per wavefront
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;  // wave-uniform on purpose
   const int c = lane % 32, h = lane / 32;
+  const int kt0 = NARROW ? (wave & 1) : 0, dt0 = NARROW ? (wave >> 1) * DTO : 0;
 
   // ---- work item: heads of a GQA group adjacent, long (late) query tiles first -------------
   int group, rank, g = 0, split = 0, item = 0;
@@ -168,7 +179,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   TileParts mine[MQ];
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
-    const int row = q0 + (wave * MQ + qt) * 32 + c;
+    const int row = q0 + (NARROW ? qt : wave * MQ + qt) * 32 + c;
     row_in[qt] = row < rows_total;
     qrow[qt] = SPLIT ? row / p.group : row;
     lane_head[qt] = SPLIT ? head + row % p.group : head;
@@ -203,14 +214,14 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   const int n_live = *live_count;
   const int i_lo = 0, i_hi = n_live;
 
-  f32x16 o[DT][MQ];
+  f32x16 o[DTO][MQ];
   float m_run[MQ], l_run[MQ];
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
     m_run[qt] = -1e30f;
     l_run[qt] = 0.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++)
+    for (int dt = 0; dt < DTO; dt++)
 #pragma unroll
       for (int i = 0; i < 16; i++) o[dt][qt][i] = 0.f;
   }
@@ -235,13 +246,13 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     const float cs = p.scale_log2;  // > 0
 
     // per-lane offsets into a swizzled tile
-    int nat_off[KSTEPS], tr_off[DT][2];
+    int nat_off[KSTEPS], tr_off[DTO][2];
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) nat_off[ks] = nat_offset<D>(c, ks, h);
 #pragma unroll
-    for (int dt = 0; dt < DT; dt++) {
-      tr_off[dt][0] = tr_offset<D>(lane, dt, 0);
-      tr_off[dt][1] = tr_offset<D>(lane, dt, 1);
+    for (int dt = 0; dt < DTO; dt++) {
+      tr_off[dt][0] = tr_offset<D>(lane, dt0 + dt, 0);
+      tr_off[dt][1] = tr_offset<D>(lane, dt0 + dt, 1);
     }
 
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
@@ -255,24 +266,29 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
                      __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + (wave & 1) * (kTK * 4)));
     };
 
-    // entries of the live list for iterations i, i + 1, i + 2 (read ahead of their use)
-    uint32_t e0 = live_list[i_lo];
-    uint32_t e1 = i_lo + 1 < i_hi ? live_list[i_lo + 1] : 0;
-    uint32_t e2 = i_lo + 2 < i_hi ? live_list[i_lo + 2] : 0;
-    issue(e0 & 0xffffff, 0);
-    if (STAGES == 3 && i_lo + 1 < i_hi) issue(e1 & 0xffffff, 1);
+    // entries of the live list for iterations i ... i + kAhead (read ahead of their use); the ring
+    // holds the tile being worked on and the kAhead tiles requested after it
+    constexpr int kAhead = STAGES - 1;
+    static_assert(kAhead >= 1 && kAhead <= 3 && kAhead * kCopies < 64, "prefetch distance");
+    uint32_t e[kAhead + 1];
+#pragma unroll
+    for (int k = 0; k <= kAhead; k++) e[k] = i_lo + k < i_hi ? live_list[i_lo + k] : 0;
+#pragma unroll
+    for (int k = 0; k < kAhead; k++)
+      if (k == 0 || i_lo + k < i_hi) issue(e[k] & 0xffffff, k);
 
     int stage = 0;
     for (int i = i_lo; i < i_hi; i++) {
-      // tile i has landed once at most the copies of tile i + 1 are outstanding
-      if (STAGES == 3 && i + 1 < i_hi) wait_vmcnt<kCopies>(); else wait_vmcnt<0>();
+      // tile i has landed once at most the copies of the tiles requested after it are outstanding
+      const int later = min(kAhead - 1, i_hi - 1 - i);
+      if (kAhead >= 3 && later >= 2) wait_vmcnt<(kAhead >= 3 ? 2 : 0) * kCopies>();
+      else if (kAhead >= 2 && later >= 1) wait_vmcnt<(kAhead >= 2 ? 1 : 0) * kCopies>();
+      else wait_vmcnt<0>();
       __syncthreads();
-      const uint32_t e3 = i + 3 < i_hi ? live_list[i + 3] : 0;
-      if (STAGES == 3) {
-        if (i + 2 < i_hi) issue(e2 & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);  // (stage + 2) % 3
-      } else {
-        if (i + 1 < i_hi) issue(e1 & 0xffffff, stage ^ 1);
-      }
+      const uint32_t e_next = i + kAhead + 1 < i_hi ? live_list[i + kAhead + 1] : 0;
+      // into the stage of tile i - 1, which every wavefront has left
+      if (i + kAhead < i_hi) issue(e[kAhead] & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);
+      const uint32_t e0 = e[0];
       const int t = e0 & 0xffffff;
 
       if ((e0 >> (24 + wave)) & 1) {
@@ -282,28 +298,28 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
         const int32_t* ids = reinterpret_cast<const int32_t*>(ktile + 2 * Smem::kTileBytes);
 
         // ---- S^T = K Q^T -----------------------------------------------------------------
-        f32x16 s[2][MQ];
+        f32x16 s[KT][MQ];  // key half kt0 + kt
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+        for (int kt = 0; kt < KT; kt++)
 #pragma unroll
           for (int qt = 0; qt < MQ; qt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) s[kt][qt][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++) {
-          vec8 a[2];
+          vec8 a[KT];
 #pragma unroll
-          for (int kt = 0; kt < 2; kt++)
-            a[kt] = *reinterpret_cast<const vec8*>(ktile + 32 * kt * RB + nat_off[ks]);
+          for (int kt = 0; kt < KT; kt++)
+            a[kt] = *reinterpret_cast<const vec8*>(ktile + 32 * (kt0 + kt) * RB + nat_off[ks]);
 #pragma unroll
-          for (int kt = 0; kt < 2; kt++)
+          for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int qt = 0; qt < MQ; qt++) s[kt][qt] = Tr::mfma(a[kt], qf[qt][ks], s[kt][qt]);
         }
         // issue order: operand reads run four ahead of the MFMAs that consume them
         __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-        for (int i = 0; i < 2 * KSTEPS - 4; i++) {
+        for (int i = 0; i < KT * KSTEPS - 4; i++) {
           __builtin_amdgcn_sched_group_barrier(0x008, MQ, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
@@ -312,20 +328,20 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
         // ---- element mask outside the full range (raw scores; masked -> -inf) -------------
         if (!(t >= tf_lo && t < tf_hi)) {
 #pragma unroll
-          for (int kt = 0; kt < 2; kt++)
+          for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int qt = 0; qt < MQ; qt++)
-              mask_c_tile<true>(s[kt][qt], ids, ids + kTK, 32 * kt, kv0, h, qseg[qt], qpos[qt],
+              mask_c_tile<true>(s[kt][qt], ids, ids + kTK, 32 * (kt0 + kt), kv0, h, qseg[qt], qpos[qt],
                                 col_lo[qt], col_width[qt], -INFINITY);
         }
 
-        vec8 pb[2][2][MQ];
+        vec8 pb[KT][2][MQ];
         // ---- online softmax (per query column = per lane, halves combined once) ------------
 #pragma unroll
         for (int qt = 0; qt < MQ; qt++) {
           float mx = s[0][qt][0];
 #pragma unroll
-          for (int kt = 0; kt < 2; kt++)
+          for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
           mx = fmaxf(mx, xor32(mx));
@@ -339,7 +355,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
             const float alpha = fast_exp2(m_run[qt] - m_new);
             l_run[qt] *= alpha;
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++)
+            for (int dt = 0; dt < DTO; dt++)
 #pragma unroll
               for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
             m_run[qt] = m_new;
@@ -347,7 +363,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           const float m_use = m_run[qt];
           float sum = 0.f;
 #pragma unroll
-          for (int kt = 0; kt < 2; kt++) {
+          for (int kt = 0; kt < KT; kt++) {
 #pragma unroll
             for (int i = 0; i < 16; i++) s[kt][qt][i] = fast_exp2(__builtin_fmaf(s[kt][qt][i], cs, -m_use));
 #pragma unroll
@@ -366,35 +382,39 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 
         // ---- O^T += V^T P^T ---------------------------------------------------------------
 #pragma unroll
-        for (int kt = 0; kt < 2; kt++)
+        for (int kt = 0; kt < KT; kt++)
 #pragma unroll
           for (int st = 0; st < 2; st++)
 #pragma unroll
-            for (int dt = 0; dt < DT; dt++) {
-              const vec8 a = tr_read_a_swz<Tr>(vtile + (32 * kt + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+            for (int dt = 0; dt < DTO; dt++) {
+              const vec8 a = tr_read_a_swz<Tr>(vtile + (32 * (kt0 + kt) + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
 #pragma unroll
               for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
             }
       }
-      e0 = e1, e1 = e2, e2 = e3;
+#pragma unroll
+      for (int k = 0; k < kAhead; k++) e[k] = e[k + 1];
+      e[kAhead] = e_next;
       stage = stage == STAGES - 1 ? 0 : stage + 1;
     }
   }
 
-  // ---- split mode with several splits: leave the unnormalised partial result ---------------
-  if (SPLIT && p.num_splits > 1) {
-    const int prow = wave * 32 + c;  // MQ == 1
+  // ---- split mode with several parts per item: leave the unnormalised partial result (narrow
+  // mode: one per key half of every window, its head-dim slices written by two wavefronts) --------
+  if (SPLIT && (NARROW || p.num_splits > 1)) {
+    const int prow = (NARROW ? 0 : wave) * 32 + c;  // MQ == 1
     const float l_row = l_run[0] + xor32(l_run[0]);  // cross-lane: outside the divergent branch
     if (row_in[0] && prow < p.part_rows) {
-      const int64_t slot = ((int64_t)item * p.num_splits + split) * p.part_rows + prow;
-      float* po = p.part_o + slot * D;
+      const int64_t part = ((int64_t)item * p.num_splits + split) * (NARROW ? 2 : 1) + kt0;
+      const int64_t slot = part * p.part_rows + prow;
+      float* po = p.part_o + slot * D + 32 * dt0;
 #pragma unroll
-      for (int dt = 0; dt < DT; dt++)
+      for (int dt = 0; dt < DTO; dt++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++)
           *reinterpret_cast<float4*>(po + 32 * dt + 8 * g4 + 4 * h) =
               make_float4(o[dt][0][4 * g4 + 0], o[dt][0][4 * g4 + 1], o[dt][0][4 * g4 + 2], o[dt][0][4 * g4 + 3]);
-      if (h == 0) *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], l_row);
+      if (h == 0 && dt0 == 0) *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], l_row);
     }
     return;
   }
@@ -409,7 +429,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       char* row = (SPLIT ? p.out + ((int64_t)b * p.o_sb + (int64_t)lane_head[qt] * p.o_sh) * 2 : obase) +
                   (int64_t)qrow[qt] * p.o_ss * 2;
 #pragma unroll
-      for (int dt = 0; dt < DT; dt++)
+      for (int dt = 0; dt < DTO; dt++)
 #pragma unroll
         for (int g4 = 0; g4 < 4; g4++) {
           uint2 u;
@@ -438,13 +458,13 @@ __global__ __launch_bounds__(D) void fa_fwd_combine_kernel(const FwdParams p, in
   const int kv_head = group % p.num_kv_heads, b = group / p.num_kv_heads;
   const int qi = row / p.group, head = kv_head * p.group + row % p.group;
   const int d = threadIdx.x;
-  const int64_t slot0 = (int64_t)item * p.num_splits * p.part_rows + prow;
+  const int64_t slot0 = (int64_t)item * p.num_parts * p.part_rows + prow;
   float m = -1e30f;
 #pragma unroll 8
-  for (int s = 0; s < p.num_splits; s++) m = fmaxf(m, p.part_ml[(slot0 + (int64_t)s * p.part_rows) * 2]);
+  for (int s = 0; s < p.num_parts; s++) m = fmaxf(m, p.part_ml[(slot0 + (int64_t)s * p.part_rows) * 2]);
   float l = 0.f, acc = 0.f;
 #pragma unroll 8
-  for (int s = 0; s < p.num_splits; s++) {
+  for (int s = 0; s < p.num_parts; s++) {
     const int64_t slot = slot0 + (int64_t)s * p.part_rows;
     const float2 ml = *reinterpret_cast<const float2*>(p.part_ml + slot * 2);
     const float w = ml.y > 0.f ? fast_exp2(ml.x - m) : 0.f;
@@ -471,6 +491,7 @@ constexpr int kSplitWorkGroups = 1024;
 struct FwdPlan {
   bool split_mode = false;
   int num_splits = 1, split_tiles = 0;
+  int num_parts = 1;  // partial results per item: twice num_splits in narrow mode (at most 32 rows)
   int part_rows = 0;
   size_t part_o_bytes = 0, part_ml_bytes = 0;
 };
@@ -492,16 +513,19 @@ FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv
   window = window > cdiv(n_kv_tiles, 64) ? window : cdiv(n_kv_tiles, 64);
   plan.split_tiles = window;
   plan.num_splits = cdiv(n_kv_tiles, window);
-  if (plan.num_splits > 1) {
+  // narrow mode (see fa_fwd_kernel) where the key sequence is divided anyway: with a single window it
+  // would only add the launch that merges the partial results
+  plan.num_parts = plan.num_splits * (rows <= 32 && plan.num_splits > 1 ? 2 : 1);
+  if (plan.num_parts > 1) {
     plan.part_rows = (int)(rows < kSplitTileRows ? rows : kSplitTileRows);
-    const size_t slots = (size_t)items * plan.num_splits * plan.part_rows;
+    const size_t slots = (size_t)items * plan.num_parts * plan.part_rows;
     plan.part_o_bytes = (slots * head_dim * sizeof(float) + 15) / 16 * 16;
     plan.part_ml_bytes = (slots * 2 * sizeof(float) + 15) / 16 * 16;
   }
   return plan;
 }
 
-template <class Tr, int D, int MQ, int NW, int WPS, int STAGES = 3, bool SPLIT = false>
+template <class Tr, int D, int MQ, int NW, int WPS, int STAGES = 3, bool SPLIT = false, bool NARROW = false>
 int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   FwdParams p = p0;
   constexpr int TQ = NW * 32 * MQ;
@@ -510,12 +534,12 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
     p.num_q_tiles = cdiv(p.q_len * p.group, TQ);
     p.total_items = p.batch * p.num_kv_heads * p.num_q_tiles * p.num_splits;
   } else {
-    p.num_splits = 1;
+    p.num_splits = p.num_parts = 1;
     p.num_q_tiles = cdiv(p.q_len, TQ);
     p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_q_tiles, p.group}.grid();
   }
   if (p.batch * p.num_heads * p.num_q_tiles == 0) return KVAX_OK;
-  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES, SPLIT>;
+  auto kernel = fa_fwd_kernel<Tr, D, MQ, NW, WPS, STAGES, SPLIT, NARROW>;
   const int smem = FwdSmem<D, STAGES>::kTotal + live_tiles_bytes(NW, p.n_kv_tiles);
   constexpr int kWgPerCu = (WPS * 4 / NW) > 0 ? (WPS * 4 / NW) : 1;
   constexpr int kMaxSmem = kLdsPerCu / kWgPerCu;
@@ -526,7 +550,7 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   if (int rc = reservation.ensure(kernel, kMaxSmem, "the forward kernel")) return rc;
   hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
   if (int rc = check_launch("fa_fwd_kernel")) return rc;
-  if (SPLIT && p.num_splits > 1) {
+  if (SPLIT && p.num_parts > 1) {
     const int blocks = p.batch * p.num_kv_heads * p.num_q_tiles * p.part_rows;
     hipLaunchKernelGGL((fa_fwd_combine_kernel<Tr, D>), dim3(blocks), dim3(D), 0, stream, p, TQ);
     return check_launch("fa_fwd_combine_kernel");
@@ -542,10 +566,12 @@ int launch_fwd_auto(const FwdParams& p, hipStream_t stream) {
   if constexpr (D == 256) {
     // 128 accumulator registers for O and 64 for the Q fragments: one wavefront per SIMD, one
     // work-group of four per compute unit, two 64.5 KB stages
+    if (p.split_mode && p.num_parts > p.num_splits) return launch_fwd<Tr, D, 1, 4, 1, 2, true, true>(p, stream);
     if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 1, 2, true>(p, stream);
     return launch_fwd<Tr, D, 1, 4, 1, 2>(p, stream);
   } else {
     constexpr int kStagesSmall = D == 128 ? 2 : 3;
+    if (p.split_mode && p.num_parts > p.num_splits) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall, true, true>(p, stream);
     if (p.split_mode) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall, true>(p, stream);
     const int small = FwdSmem<D, kStagesSmall>::kTotal + live_tiles_bytes(4, p.n_kv_tiles);
     if (small <= kLdsHalfCu) return launch_fwd<Tr, D, 1, 4, 2, kStagesSmall>(p, stream);
@@ -691,6 +717,7 @@ int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, 
     const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim);
     p.split_mode = plan.split_mode;
     p.num_splits = plan.num_splits;
+    p.num_parts = plan.num_parts;
     p.split_tiles = plan.split_tiles;
     p.part_rows = plan.part_rows;
     p.part_o = (float*)((char*)workspace + tile_summary_bytes(a->batch, a->kv_len));

@@ -279,6 +279,10 @@ def test_errors(device):
     (48, 2048, 16, 4, 128, 2, 0, 1),      # 192 rows per kv head: two row tiles
     (200, 3000, 6, 2, 64, 1, 37, 3),      # ragged prefill chunk with documents and padding
     (128, 1024, 4, 1, 128, 1, 100, 2),    # multi-query attention
+    (1, 4096, 16, 4, 256, 2, 0, 1),       # decode at head_dim 256
+    (3, 2500, 8, 1, 256, 1, 0, 2),        # 24 rows per kv head, documents, head_dim 256
+    (2, 3000, 32, 2, 64, 2, 5, 2),        # exactly 32 rows per kv head, padding, head_dim 64
+    (9, 3000, 8, 2, 128, 2, 0, 1),        # 36 rows per kv head: just beyond the 32-row case
 ])
 def test_split_mode_matches_dense_oracle(device, sq, sk, hq, hkv, d, batch, pad, nseg):
     lengths = generate_random_segments_lengths(sk, nseg)
