@@ -79,6 +79,43 @@ def parse():
     return ap.parse_args()
 
 
+def read_sclk_mhz():
+    """Current shader clock in MHz as the amdgpu driver reports it for the first card
+    (the starred line of pp_dpm_sclk), or None where the file is not there."""
+    import glob
+    import re
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            for line in open(path):
+                if line.rstrip().endswith("*"):
+                    m = re.search(r"(\d+)\s*[Mm][Hh]z", line)
+                    if m:
+                        return float(m.group(1))
+        except OSError:
+            pass
+    return None
+
+
+def sample_sclk(step, ms_per_step, seconds=0.4, samples=8):
+    """Shader clock while the timed work runs: enqueues about `seconds` of steps without waiting and
+    reads the driver's clock from the host in the meantime.  Returns (mean MHz, samples) or None."""
+    if read_sclk_mhz() is None:
+        return None
+    n = max(8, int(seconds * 1e3 / max(ms_per_step, 1e-3)))
+    n = min(n, 2000)
+    # enqueueing is much faster than the kernels run: the queue holds the work while the host samples
+    for _ in range(n):
+        step()
+    got = []
+    for i in range(samples):
+        time.sleep(seconds * 0.8 / samples)
+        v = read_sclk_mhz()
+        if v is not None and i >= 1:  # the first interval lets the clock settle
+            got.append(v)
+    torch.cuda.synchronize()
+    return (float(np.mean(got)), len(got)) if got else None
+
+
 def cpu_baseline(w, seed, seconds_hint=20.0):
     """Dense masked attention (forward + backward) on the host cores for ONE query head of the
     workload, numpy float32, row-blocked; returns the JSON object.  The oracle is the thing
@@ -224,7 +261,9 @@ def measure(args, name, block, steps, warmup, device_tensors=False):
                     "peak": MFMA_BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
                     "traffic": recorded_traffic(dominant, name)}
+    sclk = sample_sclk(step, ms_per_step) if args.workload == name else None
     figures = {
+        "sclk": sclk,
         "value": value, "ms_per_step": ms_per_step, "pairs": pairs, "f_step": f_step, "f_fwd": f_fwd,
         "roofline": roofline, "mask_build_ms": mask_ms, "kernel_ms": kernel_ms,
         "kernel_tflops": {n: (kernel_flops[n] / (ms * 1e-3) / 1e12 if ms > 0 else 0.0)
@@ -296,6 +335,11 @@ def main():
         "mask_build_ms": m["mask_build_ms"],
         "kernel_ms": m["kernel_ms"],
         "kernel_tflops": m["kernel_tflops"],
+        # the peak above assumes the datasheet's 2.4 GHz; this is the shader clock the driver reported
+        # (pp_dpm_sclk) while the same steps ran again after the timed region
+        "clock": {"assumed_by_peak_mhz": 2400.0,
+                  "under_load_mhz": m["sclk"][0] if m["sclk"] else None,
+                  "samples": m["sclk"][1] if m["sclk"] else 0},
     }
     if not args.no_secondary and args.workload == "doc32k":
         others = {}
