@@ -159,6 +159,17 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   // (reference attn_bwd_preprocess, flash_attention_triton.py:373-410), which is also written out
   // for the dK/dV kernel.
   uint4 draw[KSTEPS];
+  // Q fragments (B operand of S^T = K Q^T), requested with dO and O so that their latency does not
+  // follow that of the live-tile bookkeeping below
+  uint4 qraw[KSTEPS];
+  {
+    const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      qraw[ks] = make_uint4(0, 0, 0, 0);
+      if (in && t_hi > t_lo) qraw[ks] = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
+    }
+  }
   float delta_q = 0.f;
   {
     const char* dr = p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh + (int64_t)(in ? qrow : 0) * p.do_ss) * 2;
@@ -206,15 +217,10 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
 
   if (n_live > 0) {
     vec8 qf[KSTEPS], dof[KSTEPS];
-    {
-      const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        uint4 u = make_uint4(0, 0, 0, 0);
-        if (in) u = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
-        qf[ks] = __builtin_bit_cast(vec8, u);
-        dof[ks] = __builtin_bit_cast(vec8, draw[ks]);
-      }
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      qf[ks] = __builtin_bit_cast(vec8, qraw[ks]);
+      dof[ks] = __builtin_bit_cast(vec8, draw[ks]);
     }
     int nat_off[KSTEPS], tr_off[DT][2];
 #pragma unroll

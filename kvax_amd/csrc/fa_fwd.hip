@@ -198,6 +198,24 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     mine[qt] = wave_parts(valid && col_width[qt] > 0, qseg[qt], qpos[qt]);
   }
 
+  // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step.
+  // Requested before the live-tile bookkeeping below so that their latency runs beside it.
+  // A negative scale is folded into Q so that the softmax below can assume scale_log2 > 0.
+  vec8 qf[MQ][KSTEPS];
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    const bool in = row_in[qt] && t_hi > t_lo;  // nothing to attend to: no reads
+    const char* row = (SPLIT ? p.q + ((int64_t)b * p.q_sb + (int64_t)lane_head[qt] * p.q_sh) * 2 : qbase) +
+                      (int64_t)(in ? qrow[qt] : 0) * p.q_ss * 2;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      uint4 u = make_uint4(0, 0, 0, 0);
+      if (in) u = *reinterpret_cast<const uint4*>(row + (16 * ks + 8 * h) * 2);
+      u.x ^= p.q_sign, u.y ^= p.q_sign, u.z ^= p.q_sign, u.w ^= p.q_sign;
+      qf[qt][ks] = __builtin_bit_cast(vec8, u);
+    }
+  }
+
   // ---- live tiles: each wave marks the kv tiles of [t_lo, t_hi) its rows can interact with; the
   // union is compacted into a list the work-group then walks -------------------------------------
   int* live_count = reinterpret_cast<int*>(smem + Smem::kTotal);
@@ -227,22 +245,6 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   }
 
   if (i_hi > i_lo) {
-    // Q fragments (B operand of S^T = K Q^T): lane holds 8 consecutive head-dim elements per step.
-    // A negative scale is folded into Q so that the softmax below can assume scale_log2 > 0.
-    vec8 qf[MQ][KSTEPS];
-#pragma unroll
-    for (int qt = 0; qt < MQ; qt++) {
-      const bool in = row_in[qt];
-      const char* row = (SPLIT ? p.q + ((int64_t)b * p.q_sb + (int64_t)lane_head[qt] * p.q_sh) * 2 : qbase) +
-                        (int64_t)(in ? qrow[qt] : 0) * p.q_ss * 2;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ks++) {
-        uint4 u = make_uint4(0, 0, 0, 0);
-        if (in) u = *reinterpret_cast<const uint4*>(row + (16 * ks + 8 * h) * 2);
-        u.x ^= p.q_sign, u.y ^= p.q_sign, u.z ^= p.q_sign, u.w ^= p.q_sign;
-        qf[qt][ks] = __builtin_bit_cast(vec8, u);
-      }
-    }
     const float cs = p.scale_log2;  // > 0
 
     // per-lane offsets into a swizzled tile
