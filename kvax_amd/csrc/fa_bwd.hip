@@ -141,19 +141,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   const int t_hi = r.hi > r.lo ? (r.hi + kTile - 1) / kTile : t_lo;
   const int tf_lo = (r.flo + kTile - 1) / kTile, tf_hi = r.fhi / kTile;
 
-  // per-lane query column
+  // per-lane query column.  Its ids, its row of the block mask and lse are read without waiting
+  // for one another (index 0 stands in for rows beyond the sequence), as are dO, O, Q and the first
+  // 64 tile summaries below: one trip to memory for the whole prologue instead of several in a row.
   const int qrow = q0 + wave * 32 + c;
   const bool in = qrow < p.q_len;
-  const int qseg = in ? p.q_seg[(int64_t)b * p.q_len + qrow] : -1;
-  const int qpos = in ? p.q_pos[(int64_t)b * p.q_len + qrow] : 0;
-  int col_lo = 0;
-  unsigned col_width = 0;
-  float lse_q = 0.f;
-  if (in && qseg != -1) {
-    col_lo = p.dq_mask[0][mbase + qrow / qbs] * kbs;
-    col_width = (unsigned)max(min(p.dq_mask[1][mbase + qrow / qbs] * kbs, p.kv_len) - col_lo, 0);
-    lse_q = p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qrow];
-  }
+  const int qi = in ? qrow : 0;
+  const int qseg_raw = p.q_seg[(int64_t)b * p.q_len + qi];
+  const int qpos_raw = p.q_pos[(int64_t)b * p.q_len + qi];
+  const int lower_raw = p.dq_mask[0][mbase + qi / qbs], upper_raw = p.dq_mask[1][mbase + qi / qbs];
+  const float lse_raw = p.lse[((int64_t)b * p.num_heads + head) * p.q_len + qi];
+  const int4* kv_summaries = p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles;
+  const WordSummaries first_word = load_word_summaries(kv_summaries, t_lo >> 6, t_lo, t_hi, lane);
   // dO fragments (B operand of dP^T = V dO^T): lane holds 8 consecutive head-dim elements per
   // step, i.e. half of its row; with the same half of O they give delta = rowsum(O * dO)
   // (reference attn_bwd_preprocess, flash_attention_triton.py:373-410), which is also written out
@@ -161,27 +160,30 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   uint4 draw[KSTEPS];
   // Q fragments (B operand of S^T = K Q^T), requested with dO and O so that their latency does not
   // follow that of the live-tile bookkeeping below
-  uint4 qraw[KSTEPS];
+  uint4 qraw[KSTEPS], oraw[KSTEPS];
   {
-    const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)(in ? qrow : 0) * p.q_ss) * 2;
+    // rows beyond the sequence read row 0 and are zeroed afterwards: no load sits behind a branch
+    const char* qr = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh + (int64_t)qi * p.q_ss) * 2;
+    const char* dr = p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh + (int64_t)qi * p.do_ss) * 2;
+    const char* orow = p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh + (int64_t)qi * p.o_ss) * 2;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
-      qraw[ks] = make_uint4(0, 0, 0, 0);
-      if (in && t_hi > t_lo) qraw[ks] = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
+      draw[ks] = *reinterpret_cast<const uint4*>(dr + (16 * ks + 8 * h) * 2);
+      oraw[ks] = *reinterpret_cast<const uint4*>(orow + (16 * ks + 8 * h) * 2);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) qraw[ks] = make_uint4(0, 0, 0, 0);
+    if (t_hi > t_lo) {  // wave-uniform: nothing to attend to, no Q
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) qraw[ks] = *reinterpret_cast<const uint4*>(qr + (16 * ks + 8 * h) * 2);
     }
   }
   float delta_q = 0.f;
   {
-    const char* dr = p.dout + ((int64_t)b * p.do_sb + (int64_t)head * p.do_sh + (int64_t)(in ? qrow : 0) * p.do_ss) * 2;
-    const char* orow = p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh + (int64_t)(in ? qrow : 0) * p.o_ss) * 2;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
-      uint4 o4 = make_uint4(0, 0, 0, 0);
-      draw[ks] = o4;
-      if (in) {
-        draw[ks] = *reinterpret_cast<const uint4*>(dr + (16 * ks + 8 * h) * 2);
-        o4 = *reinterpret_cast<const uint4*>(orow + (16 * ks + 8 * h) * 2);
-      }
+      if (!in) draw[ks] = oraw[ks] = qraw[ks] = make_uint4(0, 0, 0, 0);
+      const uint4 o4 = oraw[ks];
       const uint32_t ow[4] = {o4.x, o4.y, o4.z, o4.w}, gw[4] = {draw[ks].x, draw[ks].y, draw[ks].z, draw[ks].w};
 #pragma unroll
       for (int w = 0; w < 4; w++) {
@@ -192,6 +194,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
     delta_q += xor32(delta_q);
     if (in && h == 0) p.delta[((int64_t)b * p.num_heads + head) * p.q_len + qrow] = delta_q;
   }
+  const int qseg = in ? qseg_raw : -1;
+  const int qpos = in ? qpos_raw : 0;
+  int col_lo = 0;
+  unsigned col_width = 0;
+  float lse_q = 0.f;
+  if (in && qseg != -1) {
+    col_lo = lower_raw * kbs;
+    col_width = (unsigned)max(min(upper_raw * kbs, p.kv_len) - col_lo, 0);
+    lse_q = lse_raw;
+  }
   TileParts mine[1];
   mine[0] = wave_parts(col_width > 0, qseg, qpos);
 
@@ -201,8 +213,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   const int word0 = t_lo >> 6;
   const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
   const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.n_kv_tiles, 64) + 1));
-  mark_live_tiles<true, 1>(p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles, mine, t_lo, t_hi,
-                           live_bits + wave * words, word0, lane);
+  mark_live_tiles<true, 1>(kv_summaries, mine, t_lo, t_hi, live_bits + wave * words, word0, lane, first_word);
   __syncthreads();
   if (wave == 0)
     compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
@@ -463,8 +474,9 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   // pair mark the same tiles)
   const int word0 = c_lo >> 6;
   const int words = ((c_hi - 1) >> 6) - word0 + 1;
-  mark_live_tiles<false, 1>(p.q_tiles + 2 * (int64_t)b * p.n_q_tiles, mine, c_lo, c_hi,
-                            live_bits + wave * words, word0, lane);
+  const int4* q_summaries = p.q_tiles + 2 * (int64_t)b * p.n_q_tiles;
+  mark_live_tiles<false, 1>(q_summaries, mine, c_lo, c_hi, live_bits + wave * words, word0, lane,
+                            load_word_summaries(q_summaries, word0, c_lo, c_hi, lane));
   __syncthreads();
   if (wave == 0)
     // highest query tile first: every kv work-group of a document ends on the document's last query

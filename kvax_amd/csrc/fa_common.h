@@ -169,23 +169,38 @@ __device__ __forceinline__ bool parts_cannot_attend(const TileParts& q, const Ti
          cannot_attend(q.b, k.b);
 }
 
+// Summaries of the 64 tiles of bitmap word w, one per lane (those outside [t_lo, t_hi) are not read).
+struct WordSummaries {
+  TileParts parts;
+  bool have;
+};
+__device__ __forceinline__ WordSummaries load_word_summaries(const int4* tiles, int w, int t_lo, int t_hi, int lane) {
+  WordSummaries s;
+  const int t = w * 64 + lane;
+  s.have = t >= t_lo && t < t_hi;
+  s.parts.a = s.parts.b = empty_summary();
+  if (s.have) {
+    s.parts.a = tiles[2 * t];
+    s.parts.b = tiles[2 * t + 1];
+  }
+  return s;
+}
+
 // Live-tile bitmaps.  Each wavefront marks, for the tiles [t_lo, t_hi) of the streamed axis, the
 // ones its own rows (NP parts sets) can interact with; bit t % 64 of word t / 64 - word0.
-// `bits` points at this wave's words in LDS.
+// `bits` points at this wave's words in LDS.  `first`: the summaries of word word0, which callers
+// request early, together with the other loads of their prologue.
 template <bool MINE_IS_QUERY, int NP>
 __device__ __forceinline__ void mark_live_tiles(const int4* tiles, const TileParts (&mine)[NP],
                                                 int t_lo, int t_hi, unsigned long long* bits,
-                                                int word0, int lane) {
+                                                int word0, int lane, const WordSummaries& first) {
   for (int w = word0; w * 64 < t_hi; w++) {
-    const int t = w * 64 + lane;
+    const WordSummaries other = w == word0 ? first : load_word_summaries(tiles, w, t_lo, t_hi, lane);
     bool live = false;
-    if (t >= t_lo && t < t_hi) {
-      TileParts other;
-      other.a = tiles[2 * t];
-      other.b = tiles[2 * t + 1];
+    if (other.have) {
 #pragma unroll
       for (int i = 0; i < NP; i++)
-        live |= MINE_IS_QUERY ? !parts_cannot_attend(mine[i], other) : !parts_cannot_attend(other, mine[i]);
+        live |= MINE_IS_QUERY ? !parts_cannot_attend(mine[i], other.parts) : !parts_cannot_attend(other.parts, mine[i]);
     }
     const unsigned long long m = __ballot(live);
     if (lane == 0) bits[w - word0] = m;
