@@ -64,6 +64,9 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="doc32k", choices=sorted(WORKLOAD_TEXT))
+    ap.add_argument("--no-clock-sample", action="store_true",
+                    help="skip the extra steps enqueued after the timed region to read the shader clock under "
+                         "load (keeps the launch counts of a profiler run at warmup + steps)")
     ap.add_argument("--block", type=int, default=128)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -261,7 +264,7 @@ def measure(args, name, block, steps, warmup, device_tensors=False):
                     "peak": MFMA_BF16_DENSE_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": achieved / MFMA_BF16_DENSE_PEAK_TFLOPS,
                     "traffic": recorded_traffic(dominant, name)}
-    sclk = sample_sclk(step, ms_per_step) if args.workload == name else None
+    sclk = sample_sclk(step, ms_per_step) if args.workload == name and not args.no_clock_sample else None
     figures = {
         "sclk": sclk,
         "value": value, "ms_per_step": ms_per_step, "pairs": pairs, "f_step": f_step, "f_fwd": f_fwd,

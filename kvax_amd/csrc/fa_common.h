@@ -236,6 +236,7 @@ __device__ __forceinline__ void compact_live_tiles(const unsigned long long* bit
 }
 
 // LDS of a gfx950 compute unit, and the share of each work-group when two run per compute unit.
+constexpr int kNumCus = 256;  // compute units of the part this library is built for
 constexpr int kLdsPerCu = 160 * 1024;
 constexpr int kLdsHalfCu = kLdsPerCu / 2;
 

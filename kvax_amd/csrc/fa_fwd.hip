@@ -213,7 +213,9 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     }
   }
   const int4* kv_summaries = p.kv_tiles + 2 * (int64_t)b * p.n_kv_tiles;
-  const WordSummaries first_word = load_word_summaries(kv_summaries, t_lo >> 6, t_lo, t_hi, lane);
+  // (narrow mode walks every tile of its window: see below)
+  const WordSummaries first_word =
+      load_word_summaries(kv_summaries, t_lo >> 6, t_lo, NARROW ? t_lo : t_hi, lane);
 
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
@@ -238,12 +240,22 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   const int word0 = t_lo >> 6;
   const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
   const uint32_t* live_list = reinterpret_cast<const uint32_t*>(live_bits + NW * (cdiv_dev(p.n_kv_tiles, 64) + 1));
-  mark_live_tiles<true, MQ>(kv_summaries, mine, t_lo, t_hi, live_bits + wave * words, word0, lane, first_word);
-  __syncthreads();
-  if (wave == 0)
-    compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
-  __syncthreads();
-  const int n_live = *live_count;
+  // Narrow mode (decoding) skips the bookkeeping: a window of the key cache has few dead tiles - the
+  // block mask already ends where the cache's padding begins - and the 4 us the list costs are a
+  // tenth of such a work-group's time; every tile of the window is walked by all four wavefronts,
+  // the element mask settles the rest, and the call needs no tile summaries at all.
+  if (!NARROW) {
+    mark_live_tiles<true, MQ>(kv_summaries, mine, t_lo, t_hi, live_bits + wave * words, word0, lane, first_word);
+    __syncthreads();
+    if (wave == 0)
+      compact_live_tiles<NW>(live_bits, words, word0, const_cast<uint32_t*>(live_list), live_count, lane);
+    __syncthreads();
+  }
+  const int n_live = NARROW ? max(t_hi - t_lo, 0) : *live_count;
+  // entry j of the list: tile index | mask of the wavefronts it is live for << 24
+  auto list_entry = [&](int j) -> uint32_t {
+    return NARROW ? (uint32_t)(t_lo + j) | (0xFu << 24) : live_list[j];
+  };
   const int i_lo = 0, i_hi = n_live;
 
   f32x16 o[DTO][MQ];
@@ -288,7 +300,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     static_assert(kAhead >= 1 && kAhead <= 3 && kAhead * kCopies < 64, "prefetch distance");
     uint32_t e[kAhead + 1];
 #pragma unroll
-    for (int k = 0; k <= kAhead; k++) e[k] = i_lo + k < i_hi ? live_list[i_lo + k] : 0;
+    for (int k = 0; k <= kAhead; k++) e[k] = i_lo + k < i_hi ? list_entry(i_lo + k) : 0;
 #pragma unroll
     for (int k = 0; k < kAhead; k++)
       if (k == 0 || i_lo + k < i_hi) issue(e[k] & 0xffffff, k);
@@ -301,7 +313,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       else if (kAhead >= 2 && later >= 1) wait_vmcnt<(kAhead >= 2 ? 1 : 0) * kCopies>();
       else wait_vmcnt<0>();
       __syncthreads();
-      const uint32_t e_next = i + kAhead + 1 < i_hi ? live_list[i + kAhead + 1] : 0;
+      const uint32_t e_next = i + kAhead + 1 < i_hi ? list_entry(i + kAhead + 1) : 0;
       // into the stage of tile i - 1, which every wavefront has left
       if (i + kAhead < i_hi) issue(e[kAhead] & 0xffffff, stage >= 1 ? stage - 1 : STAGES - 1);
       const uint32_t e0 = e[0];
@@ -499,11 +511,13 @@ __global__ __launch_bounds__(D) void fa_fwd_combine_kernel(const FwdParams p, in
 // How a forward call is run: in split mode (see fa_fwd_kernel) when the query sequence is shorter
 // than a work-group's 128 rows - the heads of a GQA group then fill the rows and share the key
 // tiles - or when one work-group per 128 query rows and head would occupy less than the chip's
-// 256 compute units.  The key sequence is cut into windows of at least four tiles, about 1024 over
-// the whole batch (two rounds of two work-groups per compute unit).  Depends on the shapes only, so
-// that the workspace can be sized up front.
+// 256 compute units.  The key sequence is cut into equal windows of at least four tiles, as many as
+// make one resident set of work-groups if every range were full (two work-groups per compute unit,
+// one at head_dim 256) and never more: work-groups beyond the resident set would start when the
+// first ones end and double the time of the call (measured on 8 rows x 32k keys: 408 live
+// work-groups of 64 tiles 0.162 ms, 792 of 32 tiles 0.171, 594 of 43 tiles 0.192).  Depends on the
+// shapes only, so that the workspace can be sized up front.
 constexpr int kSplitTileRows = 128;  // (query, head) rows per work-group in split mode
-constexpr int kSplitWorkGroups = 1024;
 struct FwdPlan {
   bool split_mode = false;
   int num_splits = 1, split_tiles = 0;
@@ -523,10 +537,12 @@ FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv
   plan.split_mode = true;
   const int64_t rows = (int64_t)q_len * (num_heads / num_kv_heads);
   const int64_t items = (int64_t)batch * num_kv_heads * ((rows + kSplitTileRows - 1) / kSplitTileRows);
-  // windows of one size for every item: about kSplitWorkGroups of them if every range were full
-  int window = (int)((items * n_kv_tiles + kSplitWorkGroups - 1) / kSplitWorkGroups);
+  // windows of one size for every item, at most 64 per item
+  const int64_t resident = (head_dim == 256 ? 1 : 2) * kNumCus;
+  int64_t max_splits = items >= resident ? 1 : resident / items;
+  max_splits = max_splits < 64 ? max_splits : 64;
+  int window = cdiv(n_kv_tiles, (int)max_splits);
   window = window > 4 ? window : 4;
-  window = window > cdiv(n_kv_tiles, 64) ? window : cdiv(n_kv_tiles, 64);
   plan.split_tiles = window;
   plan.num_splits = cdiv(n_kv_tiles, window);
   // narrow mode (see fa_fwd_kernel) where the key sequence is divided anyway: with a single window it
@@ -748,7 +764,7 @@ int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, 
       return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
                   a->kv_len, need, kLdsPerCu);
   }
-  {
+  if (!(p.split_mode && p.num_parts > p.num_splits)) {  // the narrow mode does not read them
     TileSummaryJob job{a->kv_pos, a->kv_seg, workspace, a->kv_len};
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
