@@ -69,6 +69,17 @@ __device__ __forceinline__ s16x4 ds_read_tr16(const void* lds_ptr) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(KVAX_LDS(lds_ptr, s16x4));
 }
 
+// LDS reads through a 32-bit LDS address held in a register: with `addr` = per-lane part + compile-time
+// constant the constant lands in the instruction's immediate offset and costs no vector add.
+template <class T>
+__device__ __forceinline__ T lds_load(uint32_t addr) {
+  return *reinterpret_cast<__attribute__((address_space(3))) const T*>(addr);
+}
+__device__ __forceinline__ s16x4 ds_read_tr16_at(uint32_t addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      reinterpret_cast<__attribute__((address_space(3))) s16x4*>(addr));
+}
+
 // v_exp_f32 / v_log_f32 without the denormal-range fix-ups of exp2f / log2f.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
@@ -390,6 +401,13 @@ __device__ __forceinline__ int tr_offset(int lane, int dt, int half) {
   const int row = 4 * (g >> 1) + (i >> 2) + 8 * half;
   const int chunk = 4 * dt + 2 * (g & 1) + ((i & 3) >> 1);
   return row * (D * 2) + ((chunk ^ swz<D>(row)) << 4) + (i & 1) * 8;
+}
+template <class Tr>
+__device__ __forceinline__ typename Tr::vec8 tr_read_a_at(uint32_t addr_lo, uint32_t addr_hi) {
+  s16x4 lo = ds_read_tr16_at(addr_lo);
+  s16x4 hi = ds_read_tr16_at(addr_hi);
+  s16x8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(typename Tr::vec8, v);
 }
 template <class Tr>
 __device__ __forceinline__ typename Tr::vec8 tr_read_a_swz(const char* tile_row0, int off_lo, int off_hi) {

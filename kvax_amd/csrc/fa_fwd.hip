@@ -19,6 +19,8 @@
 // in which no (query, key) pair can pass the element mask are dropped up front (fa_tiles.hip).
 // Short query sequences (decoding) run in a split mode that divides the key sequence over
 // work-groups and merges their partial results (see fa_fwd_kernel).
+#include <type_traits>
+
 #include "common.h"
 #include "fa_common.h"
 
@@ -273,17 +275,24 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   if (i_hi > i_lo) {
     const float cs = p.scale_log2;  // > 0
 
-    // per-lane offsets into a swizzled tile
-    int nat_off[KSTEPS], tr_off[DTO][2];
+    // per-lane LDS addresses of the operand reads in stage 0 (K rows / V rows of key half kt0): the
+    // rest of an address - stage, key half, 16-row step - is a constant of the instruction
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
+    uint32_t nat_addr[KSTEPS], tr_addr[DTO][2];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) nat_off[ks] = nat_offset<D>(c, ks, h);
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      nat_addr[ks] = smem_addr + 32 * kt0 * RB + nat_offset<D>(c, ks, h);
+      // opaque to the optimiser, which would otherwise keep the summands and add them again per read
+      // (not at head_dim 256, where the sums would not fit the register file)
+      if constexpr (D <= 128) asm volatile("" : "+v"(nat_addr[ks]));
+    }
 #pragma unroll
     for (int dt = 0; dt < DTO; dt++) {
-      tr_off[dt][0] = tr_offset<D>(lane, dt0 + dt, 0);
-      tr_off[dt][1] = tr_offset<D>(lane, dt0 + dt, 1);
+      tr_addr[dt][0] = smem_addr + Smem::kTileBytes + 32 * kt0 * RB + tr_offset<D>(lane, dt0 + dt, 0);
+      tr_addr[dt][1] = smem_addr + Smem::kTileBytes + 32 * kt0 * RB + tr_offset<D>(lane, dt0 + dt, 1);
+      if constexpr (D <= 128) asm volatile("" : "+v"(tr_addr[dt][0]), "+v"(tr_addr[dt][1]));
     }
 
-    const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
     const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
     const AsyncTileCopy<kTK, D, NW> copy_k(p.k_ss * 2, wave, lane), copy_v(p.v_ss * 2, wave, lane);
     auto issue = [&](int tile, int stage) {
@@ -305,8 +314,12 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     for (int k = 0; k < kAhead; k++)
       if (k == 0 || i_lo + k < i_hi) issue(e[k] & 0xffffff, k);
 
-    int stage = 0;
-    for (int i = i_lo; i < i_hi; i++) {
+    // One iteration: tile i of the list, held in ring stage `stage_c`.  With a two-stage ring the
+    // driver below alternates two copies of it with the stage as a compile-time constant, so that the
+    // stage's LDS base goes into the immediate offsets of the operand reads instead of costing a
+    // vector add per read (16 of the ~150 vector instructions of a tile).
+    auto iteration = [&](int i, auto stage_c) {
+      const int stage = stage_c;
       // tile i has landed once at most the copies of the tiles requested after it are outstanding
       const int later = min(kAhead - 1, i_hi - 1 - i);
       if (kAhead >= 3 && later >= 2) wait_vmcnt<(kAhead >= 3 ? 2 : 0) * kCopies>();
@@ -322,7 +335,6 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       if ((e0 >> (24 + wave)) & 1) {
         const int kv0 = t * kTK;
         const char* ktile = smem + stage * Smem::kStage;
-        const char* vtile = ktile + Smem::kTileBytes;
         const int32_t* ids = reinterpret_cast<const int32_t*>(ktile + 2 * Smem::kTileBytes);
 
         // ---- S^T = K Q^T -----------------------------------------------------------------
@@ -338,7 +350,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           vec8 a[KT];
 #pragma unroll
           for (int kt = 0; kt < KT; kt++)
-            a[kt] = *reinterpret_cast<const vec8*>(ktile + 32 * (kt0 + kt) * RB + nat_off[ks]);
+            a[kt] = lds_load<vec8>(nat_addr[ks] + stage * Smem::kStage + 32 * kt * RB);
 #pragma unroll
           for (int kt = 0; kt < KT; kt++)
 #pragma unroll
@@ -415,7 +427,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           for (int st = 0; st < 2; st++)
 #pragma unroll
             for (int dt = 0; dt < DTO; dt++) {
-              const vec8 a = tr_read_a_swz<Tr>(vtile + (32 * (kt0 + kt) + 16 * st) * RB, tr_off[dt][0], tr_off[dt][1]);
+              const uint32_t at = stage * Smem::kStage + (32 * kt + 16 * st) * RB;
+              const vec8 a = tr_read_a_at<Tr>(tr_addr[dt][0] + at, tr_addr[dt][1] + at);
 #pragma unroll
               for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
             }
@@ -423,7 +436,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 #pragma unroll
       for (int k = 0; k < kAhead; k++) e[k] = e[k + 1];
       e[kAhead] = e_next;
-      stage = stage == STAGES - 1 ? 0 : stage + 1;
+    };
+    if constexpr (STAGES == 2 && D <= 128) {  // (two copies of the body do not fit the registers at 256)
+      for (int i = i_lo; i < i_hi; i += 2) {
+        iteration(i, std::integral_constant<int, 0>{});
+        if (i + 1 < i_hi) iteration(i + 1, std::integral_constant<int, 1>{});
+      }
+    } else {
+      int stage = 0;
+      for (int i = i_lo; i < i_hi; i++) {
+        iteration(i, stage);
+        stage = stage == STAGES - 1 ? 0 : stage + 1;
+      }
     }
   }
 
