@@ -278,19 +278,27 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
     // per-lane LDS addresses of the operand reads in stage 0 (K rows / V rows of key half kt0): the
     // rest of an address - stage, key half, 16-row step - is a constant of the instruction
     const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
+    // two copies of the loop body, one per stage of a two-stage ring (they do not fit the registers at
+    // head_dim 256)
+    constexpr bool kStaticStages = STAGES == 2 && D <= 128;
+    // at head_dim 64 reads through the generic pointer measured 2 % faster: there the registers hold
+    // offsets from the start of the LDS block, not addresses
+    constexpr bool kAddresses = D >= 128;
+    const uint32_t addr0 = kAddresses ? smem_addr : 0u;
     uint32_t nat_addr[KSTEPS], tr_addr[DTO][2];
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
-      nat_addr[ks] = smem_addr + 32 * kt0 * RB + nat_offset<D>(c, ks, h);
+      nat_addr[ks] = addr0 + 32 * kt0 * RB + nat_offset<D>(c, ks, h);
       // opaque to the optimiser, which would otherwise keep the summands and add them again per read
-      // (not at head_dim 256, where the sums would not fit the register file)
-      if constexpr (D <= 128) asm volatile("" : "+v"(nat_addr[ks]));
+      // (only where the loop below exists once per stage: elsewhere a scalar stage offset is added per
+      // read anyway, and the optimiser's own choice measured better)
+      if constexpr (kStaticStages) asm volatile("" : "+v"(nat_addr[ks]));
     }
 #pragma unroll
     for (int dt = 0; dt < DTO; dt++) {
-      tr_addr[dt][0] = smem_addr + Smem::kTileBytes + 32 * kt0 * RB + tr_offset<D>(lane, dt0 + dt, 0);
-      tr_addr[dt][1] = smem_addr + Smem::kTileBytes + 32 * kt0 * RB + tr_offset<D>(lane, dt0 + dt, 1);
-      if constexpr (D <= 128) asm volatile("" : "+v"(tr_addr[dt][0]), "+v"(tr_addr[dt][1]));
+      tr_addr[dt][0] = addr0 + Smem::kTileBytes + 32 * kt0 * RB + tr_offset<D>(lane, dt0 + dt, 0);
+      tr_addr[dt][1] = addr0 + Smem::kTileBytes + 32 * kt0 * RB + tr_offset<D>(lane, dt0 + dt, 1);
+      if constexpr (kStaticStages) asm volatile("" : "+v"(tr_addr[dt][0]), "+v"(tr_addr[dt][1]));
     }
 
     const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
@@ -350,7 +358,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           vec8 a[KT];
 #pragma unroll
           for (int kt = 0; kt < KT; kt++)
-            a[kt] = lds_load<vec8>(nat_addr[ks] + stage * Smem::kStage + 32 * kt * RB);
+            a[kt] = kAddresses ? lds_load<vec8>(nat_addr[ks] + stage * Smem::kStage + 32 * kt * RB)
+                               : *reinterpret_cast<const vec8*>(ktile + 32 * kt * RB + nat_addr[ks]);
 #pragma unroll
           for (int kt = 0; kt < KT; kt++)
 #pragma unroll
@@ -428,7 +437,8 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
 #pragma unroll
             for (int dt = 0; dt < DTO; dt++) {
               const uint32_t at = stage * Smem::kStage + (32 * kt + 16 * st) * RB;
-              const vec8 a = tr_read_a_at<Tr>(tr_addr[dt][0] + at, tr_addr[dt][1] + at);
+              const vec8 a = kAddresses ? tr_read_a_at<Tr>(tr_addr[dt][0] + at, tr_addr[dt][1] + at)
+                                        : tr_read_a_swz<Tr>(smem + at, tr_addr[dt][0], tr_addr[dt][1]);
 #pragma unroll
               for (int qt = 0; qt < MQ; qt++) o[dt][qt] = Tr::mfma(a, pb[kt][st][qt], o[dt][qt]);
             }
@@ -437,7 +447,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       for (int k = 0; k < kAhead; k++) e[k] = e[k + 1];
       e[kAhead] = e_next;
     };
-    if constexpr (STAGES == 2 && D <= 128) {  // (two copies of the body do not fit the registers at 256)
+    if constexpr (kStaticStages) {
       for (int i = i_lo; i < i_hi; i += 2) {
         iteration(i, std::integral_constant<int, 0>{});
         if (i + 1 < i_hi) iteration(i + 1, std::integral_constant<int, 1>{});
