@@ -283,6 +283,9 @@ def test_errors(device):
     (3, 2500, 8, 1, 256, 1, 0, 2),        # 24 rows per kv head, documents, head_dim 256
     (2, 3000, 32, 2, 64, 2, 5, 2),        # exactly 32 rows per kv head, padding, head_dim 64
     (9, 3000, 8, 2, 128, 2, 0, 1),        # 36 rows per kv head: just beyond the 32-row case
+    (1, 300, 16, 16, 128, 40, 0, 1),      # 640 (batch, kv head) items: more than one resident set, no windows
+    (1, 700, 32, 16, 256, 20, 0, 1),      # head_dim 256: 320 items against 256 resident work-groups
+    (2, 9000, 8, 8, 64, 9, 3, 2),         # 72 items: 7 windows each
 ])
 def test_split_mode_matches_dense_oracle(device, sq, sk, hq, hkv, d, batch, pad, nseg):
     lengths = generate_random_segments_lengths(sk, nseg)
