@@ -95,7 +95,15 @@ enum {
    * untouched; dK/dV alone reuses the delta a previous call left in the same workspace. */
   KVAX_FA_SKIP_DELTA = 16,
   KVAX_FA_SKIP_DQ = 32,
-  KVAX_FA_SKIP_DKDV = 64
+  KVAX_FA_SKIP_DKDV = 64,
+  /* Forward only, a request that is ignored where it does not apply (head_dim other than 128, short
+   * query sequences): run the forward as one work-group of four wavefronts per compute unit, each
+   * wavefront with 64 query rows, so that every K / V operand read from LDS feeds two MFMAs, with
+   * the matrix and vector instructions of the loop interleaved by hand.  Same results to rounding
+   * (the running maximum is raised per 32 keys instead of per 64).  It is as fast as the default at
+   * long dense sequences and slower on document masks (its wavefronts do not skip tiles one by
+   * one); it exists to measure what halving the LDS traffic buys.  No counterpart in the reference. */
+  KVAX_FA_FWD_WIDE = 128
 };
 
 typedef struct kvax_fa_args {
@@ -138,7 +146,8 @@ typedef struct kvax_fa_args {
  * call's work on `stream`):
  *   forward:  32 bytes per 64-row kv tile and batch row (tile summaries used to skip dead tiles),
  *             plus, for short query sequences, the fp32 partial results of the work-groups that
- *             share one key sequence (a function of the shapes only);
+ *             share one key sequence (a function of the shapes only), plus, with KVAX_FA_FWD_WIDE,
+ *             the lists of live kv tiles per 256 query rows;
  *   backward: delta [batch, num_heads, q_len] fp32, the tile summaries of the kv and the query
  *             sequence, and the dispatch order of the dK/dV work items (longest first). */
 size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* args);

@@ -15,6 +15,7 @@ KVAX_MAX_MASKS = 4
 KVAX_BF16, KVAX_F16 = 0, 1
 KVAX_FA_DKDV_F32 = 1
 KVAX_FA_SKIP_DELTA, KVAX_FA_SKIP_DQ, KVAX_FA_SKIP_DKDV = 16, 32, 64
+KVAX_FA_FWD_WIDE = 128
 KVAX_FA_FWD_STATIC_MAX_WORKSPACE = 8 << 20
 
 

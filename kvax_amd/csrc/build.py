@@ -23,6 +23,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results go to ordinary vector registers (where the element-wise code reads them) also in
+    # kernels that run one wavefront per SIMD and may use the accumulation registers as well
+    "-mllvm", "-amdgpu-mfma-vgpr-form=1",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
     f"-I{ROOT / 'include'}", f"-I{CSRC}",
 ]
@@ -60,32 +63,9 @@ def build(extra_flags: list[str] | None = None, jobs: int = 4, lib: Path | None 
     return LIB
 
 
-PROBES = ["dq_accumulate_probe.hip"]
-
-
-def build_probes() -> list[Path]:
-    """Compile the stand-alone measurement programs under ``probes/`` (one executable each, next to
-    its source).  They are not part of the library: each backs a figure quoted with a design decision."""
-    outs = []
-    for src in PROBES:
-        out = CSRC / "probes" / Path(src).stem
-        cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-               "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
-               str(CSRC / "probes" / src), "-o", str(out)]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError(f"hipcc failed on {src}:\n{r.stderr}")
-        outs.append(out)
-    return outs
-
-
 if __name__ == "__main__":
     args = sys.argv[1:]
     out = None
     if args and args[0] == "-o":
         out, args = Path(args[1]), args[2:]
     print(build(args, lib=out))
-    if out is None:
-        for probe in build_probes():
-            print(probe)

@@ -70,6 +70,37 @@ inline size_t tile_summary_bytes(int batch, int len) {
 }
 
 
+// Live-tile lists, built once per call for all query heads.  For every (batch row, item of
+// `rows_per_item` = 32 * waves query rows) the kernel merges the block-mask ranges of the mask blocks
+// the item covers, tests the kv tiles of the range against the id summaries of each wavefront's 32
+// rows and writes the tiles that are live for at least one wavefront, in ascending order:
+//   list[0] = number of entries, list[1], list[2] = first tile and end of the mask-free tile range,
+//   list[4 + j] = tile index | (mask of the wavefronts it is live for) << 24
+// (what every work-group of the attention kernels would otherwise work out for itself - the same
+// list for each of the query heads).  Lists are `tile_list_stride(n_kv_tiles)` words apart.
+struct TileListJob {
+  const int32_t* q_pos;
+  const int32_t* q_seg;
+  const int32_t* mask[4];  // lower, upper, lower_full, upper_full over the query blocks, [batch, n_qblocks]
+  const void* kv_tiles;    // summaries of the kv sequence, int4 [batch, n_kv_tiles, 2]
+  uint32_t* lists;         // out: [batch, cdiv(q_len, rows_per_item), tile_list_stride]
+  int q_len, kv_len;
+  int qbs, kbs;            // block sizes of the mask along the query and the kv axis
+  int n_qblocks, n_kv_tiles;
+  int waves;               // wavefronts per item: 4 or 8
+};
+int launch_tile_lists(const TileListJob& job, int batch, hipStream_t stream);
+__host__ __device__ inline size_t tile_list_stride(int n_kv_tiles) { return (size_t)(4 + n_kv_tiles + 3) / 4 * 4; }
+inline size_t tile_list_bytes(int batch, int q_len, int rows_per_item, int kv_len) {
+  return (size_t)batch * cdiv(q_len, rows_per_item) * tile_list_stride(cdiv(kv_len, kTileRows)) * sizeof(uint32_t);
+}
+// Above this size the lists are not built and the attention kernels fall back to working them out in
+// LDS per work-group (the size grows with q_len * kv_len / 8192 * 4 bytes: 0.5 MB for 32k x 32k).
+#ifndef KVAX_MAX_TILE_LIST_MB
+#define KVAX_MAX_TILE_LIST_MB 64
+#endif
+constexpr size_t kMaxTileListBytes = (size_t)KVAX_MAX_TILE_LIST_MB << 20;
+
 // Work-item ordering.  A work item is `sub` consecutive tiles of one sequence (the rows one
 // work-group owns); its work is the number of tiles of the other sequence that at least one of its
 // tiles can interact with according to the summaries.  Writes, per batch row, the dispatch order of

@@ -12,6 +12,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 namespace kvax {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -87,6 +90,37 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 __device__ __forceinline__ int cdiv_dev(int a, int b) { return (a + b - 1) / b; }
 
 __device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32); }
+
+// max / sum of a value with the one held by lane ^ 32, through v_permlane32_swap_b32 (exchanges
+// the upper half of one register with the lower half of another): one vector instruction where
+// __shfl_xor goes through the LDS crossbar and makes the wave wait for its answer.
+__device__ __forceinline__ void swap_halves(float x, float& a, float& b) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const unsigned r0 = r[0], r1 = r[1];  // [x.lo, x.lo] and [x.hi, x.hi]
+  a = __builtin_bit_cast(float, r0);
+  b = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float max_xor32(float x) {
+  float a, b;
+  swap_halves(x, a, b);
+  return __builtin_fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_xor32(float x) {
+  float a, b;
+  swap_halves(x, a, b);
+  return a + b;
+}
+
+// Compile-time loop: f(std::integral_constant<int, 0>) ... f(std::integral_constant<int, N - 1>).
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 // Work distribution.  Work-groups are dealt round-robin to the 8 XCDs (work-group L runs on XCD
 // L % 8, each XCD has its own L2), so the map from L to a work item decides both L2 sharing and
@@ -348,35 +382,63 @@ struct AsyncTileCopy {
   static constexpr int kPerWave = kCopies / NW;
   static constexpr int kChunks = D / 8;
   static_assert(kCopies % NW == 0, "copies must split evenly over the waves");
-  uint32_t lane_off[kPerWave];  // (row of the lane within the tile) * stride + chunk * 16, per copy
+  // Copy j of a wave covers the rows (j * NW + wave) * kRowsPerCopy + [0, kRowsPerCopy).  Up to
+  // head_dim 128 and with a multiple of four waves the swizzle term of a lane is the same in all of
+  // them, so one per-lane offset serves every copy and the scalar base moves on instead (vector
+  // registers are what the kernels run out of first).
+  static constexpr bool kCompact = D <= 128 && NW % 4 == 0;
+  static constexpr int kOffsets = kCompact ? 1 : kPerWave;
+  uint32_t lane_off[kOffsets];  // (row of the lane within the tile) * stride + chunk * 16, per copy
   int64_t stride;
-  int wave_u, rin, pos;
+  int wave_u, lane_;
 
   // The whole tile must span less than 4 GiB (ROWS * row_stride_bytes < 2^32; the entry points
   // check it), so that one scalar base per tile plus 32-bit lane offsets address every copy.
   __device__ __forceinline__ AsyncTileCopy(int64_t row_stride_bytes, int wave, int lane)
-      : stride(row_stride_bytes), wave_u(__builtin_amdgcn_readfirstlane(wave)), rin(lane / kChunks),
-        pos(lane % kChunks) {
+      : stride(row_stride_bytes), wave_u(__builtin_amdgcn_readfirstlane(wave)), lane_(lane) {
+    const int rin = lane / kChunks, pos = lane % kChunks;
 #pragma unroll
-    for (int j = 0; j < kPerWave; j++) {
+    for (int j = 0; j < kOffsets; j++) {
       const int r = (j * NW + wave_u) * kRowsPerCopy + rin;
       lane_off[j] = (uint32_t)(r * row_stride_bytes) + (uint32_t)((pos ^ swz<D>(r)) * 16);
     }
   }
 
   __device__ __forceinline__ void operator()(const char* gbase, int row0, int limit, uint32_t tile_addr) const {
-    if (row0 + ROWS <= limit) {  // whole tile in range (uniform): one scalar base + fixed lane offsets
-      const char* tile_base = gbase + (int64_t)row0 * stride;
+    part<0, kPerWave>(gbase, row0, limit, tile_addr);
+  }
+  // Rows [row0 + HF * ROWS / 2, + ROWS / 2) of the tile only, into their place in the tile at
+  // `tile_addr` (the copies of a wave alternate over groups of rows, the first half of them lies in
+  // the first half of the tile).
+  template <int HF>
+  __device__ __forceinline__ void half(const char* gbase, int row0, int limit, uint32_t tile_addr) const {
+    static_assert(kPerWave % 2 == 0, "a wave's copies must split over the two halves of a tile");
+    part<HF * (kPerWave / 2), (HF + 1) * (kPerWave / 2)>(gbase, row0, limit, tile_addr);
+  }
+  // row0 < limit
+  template <int J0, int J1>
+  __device__ __forceinline__ void part(const char* gbase, int row0, int limit, uint32_t tile_addr) const {
+    const char* tile_base = gbase + (int64_t)row0 * stride;
+    if (row0 + ROWS <= limit) {  // whole tile in range (uniform): scalar bases + fixed lane offsets
       const uint32_t lds = tile_addr + wave_u * 1024;
 #pragma unroll
-      for (int j = 0; j < kPerWave; j++) async_copy_b128(tile_base, lane_off[j], lds + j * NW * 1024);
-    } else {  // ragged tail: clamp each lane's row
+      for (int j = J0; j < J1; j++) {
+        if constexpr (kCompact)
+          async_copy_b128(tile_base + j * (NW * kRowsPerCopy) * stride, lane_off[0], lds + j * NW * 1024);
+        else
+          async_copy_b128(tile_base, lane_off[j], lds + j * NW * 1024);
+      }
+    } else {  // ragged tail: clamp each lane's row (32-bit offsets from the tile's base)
+      int l = lane_;
+      asm volatile("" : "+v"(l));  // keeps what follows from being computed ahead of a loop around the call
+      const int rin = l / kChunks, pos = l % kChunks;
+      const int last = limit - 1 - row0;
 #pragma unroll
-      for (int j = 0; j < kPerWave; j++) {
+      for (int j = J0; j < J1; j++) {
         const int grp = j * NW + wave_u;
         const int r = grp * kRowsPerCopy + rin;
-        const int grow = min(row0 + r, limit - 1);
-        async_copy_b128(gbase + (int64_t)grow * stride + (pos ^ swz<D>(r)) * 16, tile_addr + grp * 1024);
+        const uint32_t off = (uint32_t)min(r, last) * (uint32_t)stride + (uint32_t)((pos ^ swz<D>(r)) * 16);
+        async_copy_b128(tile_base, off, tile_addr + grp * 1024);
       }
     }
   }

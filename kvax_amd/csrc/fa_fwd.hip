@@ -55,6 +55,8 @@ struct FwdParams {
   int num_q_tiles, total_items;
   const int4* kv_tiles;  // tile summaries [batch, n_kv_tiles]
   int n_kv_tiles;
+  const uint32_t* lists;  // wide kernel: live-tile lists of its query tiles (see TileListJob)
+  int list_stride;        // words between two lists
   uint32_t q_sign;       // 0x80008000 when the scale is negative: Q is negated on load
   float scale_log2;      // |scale| * log2(e), > 0
   // split mode (short query sequences, see fa_fwd_kernel): rows are (query, head of the group)
@@ -311,6 +313,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
                      __builtin_amdgcn_readfirstlane(base + 2 * Smem::kTileBytes + (wave & 1) * (kTK * 4)));
     };
 
+    {
     // entries of the live list for iterations i ... i + kAhead (read ahead of their use); the ring
     // holds the tile being worked on and the kAhead tiles requested after it
     constexpr int kAhead = STAGES - 1;
@@ -393,7 +396,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
           for (int kt = 0; kt < KT; kt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[kt][qt][i]);
+#ifdef KVAX_FWD_BPERMUTE
           mx = fmaxf(mx, xor32(mx));
+#else
+          mx = max_xor32(mx);
+#endif
           // The running maximum only has to bound the scores loosely: it is raised (and O, l
           // rescaled: 64 multiplies per lane) only when some row's maximum has grown by more than
           // kRescaleStep, i.e. the exponentials below may reach 2^kRescaleStep instead of 1 - exact
@@ -459,6 +466,7 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
         stage = stage == STAGES - 1 ? 0 : stage + 1;
       }
     }
+    }
   }
 
   // ---- split mode with several parts per item: leave the unnormalised partial result (narrow
@@ -476,7 +484,11 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
         for (int g4 = 0; g4 < 4; g4++)
           *reinterpret_cast<float4*>(po + 32 * dt + 8 * g4 + 4 * h) =
               make_float4(o[dt][0][4 * g4 + 0], o[dt][0][4 * g4 + 1], o[dt][0][4 * g4 + 2], o[dt][0][4 * g4 + 3]);
-      if (h == 0 && dt0 == 0) *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], l_row);
+      // a row that may attend to nothing (padding) leaves an empty partial: its accumulator is not zero
+      // when the block mask declares padding-against-padding blocks mask-free (masks built without
+      // skipping padding), where the element mask, which is what excludes such rows, is not applied
+      if (h == 0 && dt0 == 0)
+        *reinterpret_cast<float2*>(p.part_ml + slot * 2) = make_float2(m_run[0], col_width[0] > 0 ? l_row : 0.f);
     }
     return;
   }
@@ -502,6 +514,364 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
       if (h == 0)
         (SPLIT ? p.lse + ((int64_t)b * p.num_heads + lane_head[qt]) * p.q_len : lse)[qrow[qt]] =
             alive ? m_run[qt] + fast_log2(l) : 0.f;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wide forward kernel: four wavefronts, one per SIMD, each with 64 query rows (two 32-row
+// sub-tiles) of one (batch, head), i.e. 256 query rows per work-group and one work-group per
+// compute unit.  Every K / V operand read from LDS feeds two MFMAs (one per sub-tile): reading 1 KiB
+// of LDS per MFMA, as the 32-row kernels do, caps the matrix pipeline at about 70 % whatever else
+// the wavefronts do, because the LDS delivers about 100 bytes per clock and compute unit.  With one
+// wavefront per SIMD nobody else fills the gaps in a wavefront's instruction stream, so the loop
+// is software-pipelined over half tiles of 32 keys and the order is written out: while the vector
+// unit does the softmax of half j (scores computed one half step earlier), the matrix pipeline
+// computes the scores of half j + 1 and, as the exponentials arrive, O^T += V^T P^T of half j -
+// chunks of one MFMA, its share of the operand reads and four vector instructions, kept in place
+// by scheduling fences (and, for instructions without side effects, by empty asm statements that
+// use their results).
+// Ring protocol (one barrier per tile, two stages): iteration i works on the second half of K(i),
+// the first half of K(i + 1) and all of V(i); after the barrier at its top the copies of the second
+// half of K(i + 1), of V(i + 1) with its ids and of the first half of K(i + 2) are issued into the
+// rows nobody reads any more.  One loop body serves both stages: the registers that hold the operand
+// addresses are moved to the other stage once per tile, everything else is an immediate offset.
+// Every wavefront works on every tile of the work-group's list (built by launch_tile_lists for
+// items of 256 rows): a tile that is live for another wavefront only lies outside the mask-free
+// range, so the element mask turns all of its scores into -inf and P into zeros.
+// ---------------------------------------------------------------------------------------------
+template <class Tr, int D>
+__global__ __launch_bounds__(256, 1) void fa_fwd_wide_kernel(const FwdParams p) {
+  using vec8 = typename Tr::vec8;
+  constexpr int NW = 4, MQ = 2, STAGES = 2;
+  using Smem = FwdSmem<D, STAGES>;
+  constexpr int TQ = NW * 32 * MQ;
+  constexpr int KSTEPS = D / 16, DT = D / 32, RB = D * 2;
+  constexpr int kCopies = 2 * async_tile_copies_per_wave<kTK, D, NW>() + 1;
+  static_assert(KSTEPS == 8 && DT == 4, "the chunk plan below is laid out for head_dim 128");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64), lane = tid % 64;
+  const int c = lane % 32, h = lane / 32;
+  int group, rank, g;
+  const ItemMap items{p.batch * p.num_kv_heads, p.num_q_tiles, p.group};
+  if (!items.decode(blockIdx.x, group, rank, g)) return;
+  const int q_tile = p.num_q_tiles - 1 - rank;
+  const int kv_head = group % p.num_kv_heads, b = group / p.num_kv_heads;
+  const int head = kv_head * p.group + g;
+  const int q0 = q_tile * TQ;
+
+  const int32_t* kv_seg = p.kv_seg + (int64_t)b * p.kv_len;
+  const int32_t* kv_pos = p.kv_pos + (int64_t)b * p.kv_len;
+  const char* qbase = p.q + ((int64_t)b * p.q_sb + (int64_t)head * p.q_sh) * 2;
+  const char* kbase = p.k + ((int64_t)b * p.k_sb + (int64_t)kv_head * p.k_sh) * 2;
+  const char* vbase = p.v + ((int64_t)b * p.v_sb + (int64_t)kv_head * p.v_sh) * 2;
+  char* obase = p.out + ((int64_t)b * p.o_sb + (int64_t)head * p.o_sh) * 2;
+  float* lse = p.lse + ((int64_t)b * p.num_heads + head) * p.q_len;
+
+  const uint32_t* list = p.lists + ((int64_t)b * p.num_q_tiles + q_tile) * p.list_stride;
+  const int n_live = (int)list[0], tf_lo = (int)list[1], tf_hi = (int)list[2];
+
+  // ---- per-lane query columns (sub-tile qt: rows q0 + 64 * wave + 32 * qt + c) -----------------
+  int qrow[MQ], qseg[MQ], qpos[MQ], col_lo[MQ];
+  bool row_in[MQ];
+  unsigned col_width[MQ];
+  vec8 qf[MQ][KSTEPS];
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    qrow[qt] = q0 + (wave * MQ + qt) * 32 + c;
+    row_in[qt] = qrow[qt] < p.q_len;
+    const int qi = row_in[qt] ? qrow[qt] : 0;
+    const int seg = p.q_seg[(int64_t)b * p.q_len + qi], pos = p.q_pos[(int64_t)b * p.q_len + qi];
+    const int64_t mi = (int64_t)b * p.n_qblocks + qi / p.qbs;
+    const int lower_raw = p.lower[mi], upper_raw = p.upper[mi];
+    const char* row = qbase + (int64_t)qi * p.q_ss * 2;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      uint4 u = make_uint4(0, 0, 0, 0);
+      if (row_in[qt]) u = *reinterpret_cast<const uint4*>(row + (16 * ks + 8 * h) * 2);
+      u.x ^= p.q_sign, u.y ^= p.q_sign, u.z ^= p.q_sign, u.w ^= p.q_sign;
+      // The fragments are only ever MFMA operands, which may come from the accumulation registers: put
+      // them there for good (the vector registers are needed for the scores; left to itself the
+      // register allocator parks the fragments in accumulation registers anyway, but copies them back
+      // in front of every use).
+      uint32_t a0, a1, a2, a3;
+      asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(a0) : "v"(u.x));
+      asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(a1) : "v"(u.y));
+      asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(a2) : "v"(u.z));
+      asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(a3) : "v"(u.w));
+      qf[qt][ks] = __builtin_bit_cast(vec8, make_uint4(a0, a1, a2, a3));
+    }
+    qseg[qt] = row_in[qt] ? seg : -1;
+    qpos[qt] = row_in[qt] ? pos : 0;
+    col_lo[qt] = 0;
+    col_width[qt] = 0;
+    if (row_in[qt] && seg != -1) {
+      col_lo[qt] = lower_raw * p.kbs;
+      col_width[qt] = (unsigned)max(min(upper_raw * p.kbs, p.kv_len) - col_lo[qt], 0);
+    }
+  }
+
+  f32x16 o[DT][MQ];
+  float m_run[MQ], l_run[MQ];
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    m_run[qt] = -1e30f;
+    l_run[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) o[dt][qt][i] = 0.f;
+  }
+
+  if (n_live > 0) {
+    const float cs = p.scale_log2;  // > 0
+    const uint32_t smem_addr = (uint32_t)(uintptr_t)smem;
+    uint32_t nat_addr[KSTEPS], tr_addr[DT][2];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) nat_addr[ks] = smem_addr + nat_offset<D>(c, ks, h);
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      tr_addr[dt][0] = smem_addr + Smem::kTileBytes + tr_offset<D>(lane, dt, 0);
+      tr_addr[dt][1] = smem_addr + Smem::kTileBytes + tr_offset<D>(lane, dt, 1);
+    }
+    const int32_t* id_src = (wave & 1) ? kv_pos : kv_seg;
+    const AsyncTileCopy<kTK, D, NW> copy_k(p.k_ss * 2, wave, lane), copy_v(p.v_ss * 2, wave, lane);
+    constexpr uint32_t kHalf = 32 * RB;  // bytes of 32 rows of a tile
+    auto k_read = [&](int ks, uint32_t off) { return lds_load<vec8>(nat_addr[ks] + off); };
+    auto v_read = [&](int dt, uint32_t off) { return tr_read_a_at<Tr>(tr_addr[dt][0] + off, tr_addr[dt][1] + off); };
+#define KVAX_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define KVAX_ANCHOR(x) asm volatile("" : "+v"(x))
+
+    // scores of 32 keys on their own (the first half of the first tile)
+    auto scores_only = [&](f32x16 (&nxt)[MQ]) __attribute__((always_inline)) {
+      f32x16 z;
+#pragma unroll
+      for (int i = 0; i < 16; i++) z[i] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        const vec8 a = k_read(ks, 0);
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++) nxt[qt] = Tr::mfma(a, qf[qt][ks], ks == 0 ? z : nxt[qt]);
+      }
+    };
+
+    // One half step.  cur: scores of this half (in), nxt: scores of the next half (out); voff: byte
+    // offset of this half's V rows from where the V address registers point (the K address registers
+    // point at the next half's rows).
+    auto half_step = [&](f32x16 (&cur)[MQ], f32x16 (&nxt)[MQ], auto voff_c) __attribute__((always_inline)) {
+      constexpr uint32_t voff = decltype(voff_c)::value;
+      vec8 kop[KSTEPS], vop[2 * DT];
+      uint32_t w[MQ][8];
+      float sum0[MQ], sum1[MQ];
+      // operand r of the half step's MFMA pairs: K rows of the next half (r < 8), then V^T of this
+      // half (16-key step (r - 8) / 4, head-dim block (r - 8) % 4); read kAheadOps pairs ahead
+      constexpr int kAheadOps = 3;
+      auto read_operand = [&](auto r_c) __attribute__((always_inline)) {
+        constexpr int r = decltype(r_c)::value;
+        if constexpr (r < KSTEPS) kop[r] = k_read(r, 0);
+        else if constexpr (r < KSTEPS + 2 * DT)
+          vop[r - KSTEPS] = v_read((r - KSTEPS) % DT, voff + ((r - KSTEPS) / DT) * 16 * RB);
+      };
+      static_for<kAheadOps>([&](auto r_c) __attribute__((always_inline)) { read_operand(r_c); });
+      KVAX_FENCE();
+      // ---- row maxima of both sub-tiles, with the first score MFMAs of the next half behind them
+      float mx[MQ];
+      f32x16 z;
+#pragma unroll
+      for (int i = 0; i < 16; i++) z[i] = 0.f;
+#pragma unroll
+      for (int qt = 0; qt < MQ; qt++) {
+        mx[qt] = __builtin_fmaxf(cur[qt][0], cur[qt][1]);
+#pragma unroll
+        for (int i = 2; i < 8; i += 2) mx[qt] = __builtin_fmaxf(__builtin_fmaxf(mx[qt], cur[qt][i]), cur[qt][i + 1]);
+        nxt[qt] = Tr::mfma(kop[0], qf[qt][0], z);
+        KVAX_ANCHOR(nxt[qt]);
+        if (qt == 1) read_operand(std::integral_constant<int, kAheadOps>{});
+        KVAX_FENCE();
+      }
+#pragma unroll
+      for (int qt = 0; qt < MQ; qt++) {
+#pragma unroll
+        for (int i = 8; i < 16; i += 2) mx[qt] = __builtin_fmaxf(__builtin_fmaxf(mx[qt], cur[qt][i]), cur[qt][i + 1]);
+        nxt[qt] = Tr::mfma(kop[1], qf[qt][1], nxt[qt]);
+        KVAX_ANCHOR(nxt[qt]);
+        if (qt == 1) read_operand(std::integral_constant<int, kAheadOps + 1>{});
+        KVAX_FENCE();
+      }
+#pragma unroll
+      for (int qt = 0; qt < MQ; qt++) mx[qt] = max_xor32(mx[qt]) * cs;
+      // lazy running maxima (see fa_fwd_kernel): one test for both sub-tiles
+      if (__any(mx[0] > m_run[0] + kRescaleStep || mx[1] > m_run[1] + kRescaleStep)) {
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++) {
+          const float m_new = fmaxf(m_run[qt], mx[qt]);
+          const float alpha = fast_exp2(m_run[qt] - m_new);
+          l_run[qt] *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[dt][qt][i] *= alpha;
+          m_run[qt] = m_new;
+        }
+      }
+      const float m_use[MQ] = {m_run[0], m_run[1]};
+      // vector instruction I of the 112 that turn the 2 x 16 scores into P (packed in w) and its row
+      // sums: per group of 8 elements and sub-tile 4 x (fma, fma, exp, exp) then 4 packs - group 0 of
+      // both sub-tiles, then group 1 -, and the 2 x 14 additions last
+      auto valu_op = [&](auto i_c) __attribute__((always_inline)) {
+        constexpr int I = decltype(i_c)::value;
+        if constexpr (I < 80) {
+          constexpr int grp = I / 40, qt = (I % 40) / 20, k = I % 20;
+          if constexpr (k < 16) {
+            constexpr int e = 8 * grp + 2 * (k / 4) + k % 2;
+            if constexpr (k % 4 < 2) cur[qt][e] = __builtin_fmaf(cur[qt][e], cs, -m_use[qt]);
+            else cur[qt][e] = fast_exp2(cur[qt][e]);
+          } else {
+            constexpr int j = 4 * grp + (k - 16);
+            w[qt][j] = Tr::pack2(cur[qt][2 * j], cur[qt][2 * j + 1]);
+          }
+        } else if constexpr (I < 108) {
+          constexpr int qt = (I - 80) / 14, e = (I - 80) % 14 + 2;
+          if constexpr (e == 2) sum0[qt] = cur[qt][0] + cur[qt][2];
+          else if constexpr (e == 3) sum1[qt] = cur[qt][1] + cur[qt][3];
+          else if constexpr (e % 2 == 0) sum0[qt] += cur[qt][e];
+          else sum1[qt] += cur[qt][e];
+          if constexpr (I % 4 == 3) asm volatile("" : "+v"(sum0[qt]), "+v"(sum1[qt]));  // stay in this chunk
+        }
+      };
+      // ---- chunks: MFMA pair index m = 2 .. 15 (scores of the next half up to 7, then O^T += V^T P^T
+      // of this half), two chunks (one per sub-tile) each
+      static_for<28>([&](auto c_c) __attribute__((always_inline)) {
+        constexpr int ch = decltype(c_c)::value;
+        constexpr int m = ch / 2 + 2, qt = ch % 2;
+        if constexpr (m < KSTEPS) {
+          nxt[qt] = Tr::mfma(kop[m], qf[qt][m], nxt[qt]);
+          KVAX_ANCHOR(nxt[qt]);
+        } else {
+          constexpr int st = (m - 8) / DT, dt = (m - 8) % DT;
+          const vec8 pb = __builtin_bit_cast(vec8, make_uint4(w[qt][4 * st], w[qt][4 * st + 1], w[qt][4 * st + 2], w[qt][4 * st + 3]));
+          o[dt][qt] = Tr::mfma(vop[m - 8], pb, o[dt][qt]);
+        }
+        if constexpr (qt == 1) read_operand(std::integral_constant<int, m + kAheadOps>{});
+        static_for<4>([&](auto j_c) __attribute__((always_inline)) {
+          valu_op(std::integral_constant<int, 4 * ch + decltype(j_c)::value>{});
+        });
+        KVAX_FENCE();
+      });
+#pragma unroll
+      for (int qt = 0; qt < MQ; qt++) l_run[qt] += sum0[qt] + sum1[qt];  // per half-wave partial
+    };
+
+    f32x16 sa[MQ], sb[MQ];  // scores of the first / second 32 keys of a tile
+#pragma unroll
+    for (int qt = 0; qt < MQ; qt++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) sb[qt][i] = 0.f;
+    uint32_t e0 = list[4], e1 = 1 < n_live ? list[5] : 0, e2 = 2 < n_live ? list[6] : 0;
+    // prologue: first half of K(0), scores of the first 32 keys
+    copy_k.template half<0>(kbase, (int)(e0 & 0xffffff) * kTK, p.kv_len, smem_addr);
+    {
+      const int tile = e0 & 0xffffff;
+      copy_k.template half<1>(kbase, tile * kTK, p.kv_len, smem_addr);
+      copy_v(vbase, tile * kTK, p.kv_len, smem_addr + Smem::kTileBytes);
+      async_copy_b32(id_src + min(tile * kTK + lane, p.kv_len - 1),
+                     __builtin_amdgcn_readfirstlane(smem_addr + 2 * Smem::kTileBytes + (wave & 1) * (kTK * 4)));
+      if (1 < n_live) copy_k.template half<0>(kbase, (int)(e1 & 0xffffff) * kTK, p.kv_len, smem_addr + Smem::kStage);
+    }
+    // the first copies issued have landed: first half of K(0)
+    if (1 < n_live) wait_vmcnt<kCopies>(); else wait_vmcnt<kCopies - async_tile_copies_per_wave<kTK, D, NW>() / 2>();
+    __syncthreads();
+    scores_only(sa);
+    // The K address registers point at the second half of the iteration's own stage in its first half
+    // step and at the first half of the other stage in its second; the V address registers at the
+    // iteration's stage.  The updates are made opaque to the optimiser, which would otherwise keep the
+    // first values and add the running offset again in front of every read.
+    int to_other = Smem::kStage;  // from the stage of this iteration to the other one
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      nat_addr[ks] += kHalf;
+      asm volatile("" : "+v"(nat_addr[ks]));
+    }
+    using Z = std::integral_constant<uint32_t, 0>;
+    using H = std::integral_constant<uint32_t, kHalf>;
+
+#pragma unroll 1
+    for (int i = 0; i < n_live; i++) {
+      // K(i), the first half of K(i + 1), V(i) have landed; everybody is done with iteration i - 1
+      wait_vmcnt<0>();
+      __syncthreads();
+      const uint32_t e3 = i + 3 < n_live ? list[4 + i + 3] : 0;
+      {
+        const uint32_t mine = smem_addr + (to_other < 0 ? Smem::kStage : 0), other = mine + to_other;
+        if (i + 1 < n_live) {
+          const int tile = e1 & 0xffffff;
+          copy_k.template half<1>(kbase, tile * kTK, p.kv_len, other);
+          copy_v(vbase, tile * kTK, p.kv_len, other + Smem::kTileBytes);
+          async_copy_b32(id_src + min(tile * kTK + lane, p.kv_len - 1),
+                         __builtin_amdgcn_readfirstlane(other + 2 * Smem::kTileBytes + (wave & 1) * (kTK * 4)));
+        }
+        if (i + 2 < n_live) copy_k.template half<0>(kbase, (int)(e2 & 0xffffff) * kTK, p.kv_len, mine);
+      }
+      const int t = e0 & 0xffffff;
+      const int kv0 = t * kTK;
+      const int32_t* ids = reinterpret_cast<const int32_t*>(smem + (to_other < 0 ? Smem::kStage : 0) + 2 * Smem::kTileBytes);
+      const bool full = t >= tf_lo && t < tf_hi;
+      if (!full) {
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++)
+          mask_c_tile<true>(sa[qt], ids, ids + kTK, 0, kv0, h, qseg[qt], qpos[qt], col_lo[qt], col_width[qt], -INFINITY);
+      }
+      half_step(sa, sb, Z{});  // K: second half of this stage
+      // K addresses: to the first half of the other stage
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        nat_addr[ks] += to_other - (int)kHalf;
+        asm volatile("" : "+v"(nat_addr[ks]));
+      }
+      if (!full) {
+#pragma unroll
+        for (int qt = 0; qt < MQ; qt++)
+          mask_c_tile<true>(sb[qt], ids, ids + kTK, 32, kv0, h, qseg[qt], qpos[qt], col_lo[qt], col_width[qt], -INFINITY);
+      }
+      half_step(sb, sa, H{});  // (the scores computed here are not used after the last tile)
+      // ... to its second half, and the V addresses to the other stage, for the next iteration
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ks++) {
+        nat_addr[ks] += kHalf;
+        asm volatile("" : "+v"(nat_addr[ks]));
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) {
+        tr_addr[dt][0] += to_other, tr_addr[dt][1] += to_other;
+        asm volatile("" : "+v"(tr_addr[dt][0]), "+v"(tr_addr[dt][1]));
+      }
+      to_other = -to_other;
+      e0 = e1, e1 = e2, e2 = e3;
+    }
+#undef KVAX_FENCE
+#undef KVAX_ANCHOR
+  }
+
+  // ---- epilogue: normalise, write O (query dtype) and lse ----------------------------------------
+#pragma unroll
+  for (int qt = 0; qt < MQ; qt++) {
+    const float l = sum_xor32(l_run[qt]);
+    const bool alive = l > 0.f && col_width[qt] > 0;  // padding / out-of-range rows stay zero
+    const float inv = alive ? 1.f / l : 0.f;
+    if (row_in[qt]) {
+      char* row = obase + (int64_t)qrow[qt] * p.o_ss * 2;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          uint2 u;
+          u.x = Tr::pack2(o[dt][qt][4 * g4 + 0] * inv, o[dt][qt][4 * g4 + 1] * inv);
+          u.y = Tr::pack2(o[dt][qt][4 * g4 + 2] * inv, o[dt][qt][4 * g4 + 3] * inv);
+          *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
+        }
+      if (h == 0) lse[qrow[qt]] = alive ? m_run[qt] + fast_log2(l) : 0.f;
     }
   }
 }
@@ -552,23 +922,41 @@ __global__ __launch_bounds__(D) void fa_fwd_combine_kernel(const FwdParams p, in
 // work-groups of 64 tiles 0.162 ms, 792 of 32 tiles 0.171, 594 of 43 tiles 0.192).  Depends on the
 // shapes only, so that the workspace can be sized up front.
 constexpr int kSplitTileRows = 128;  // (query, head) rows per work-group in split mode
+constexpr int kWideTileRows = 256;   // query rows per work-group of fa_fwd_wide_kernel
 struct FwdPlan {
   bool split_mode = false;
   int num_splits = 1, split_tiles = 0;
   int num_parts = 1;  // partial results per item: twice num_splits in narrow mode (at most 32 rows)
   int part_rows = 0;
   size_t part_o_bytes = 0, part_ml_bytes = 0;
+  // workspace layout: tile summaries of the kv sequence (not in narrow mode, which walks every tile
+  // of its windows), the partial results of the split mode, the live-tile lists of the wide kernel
+  bool narrow() const { return num_parts > num_splits; }
+  bool wide = false;  // regular mode with fa_fwd_wide_kernel (on request): lists for items of 256 query rows
+  size_t summary_bytes = 0, list_bytes = 0;
+  size_t total_bytes() const { return summary_bytes + part_o_bytes + part_ml_bytes + list_bytes; }
 };
-FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv_heads, int head_dim) {
+FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv_heads, int head_dim,
+                     bool want_wide) {
   FwdPlan plan;
   if (batch <= 0 || q_len <= 0 || kv_len <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads) return plan;
   const int n_kv_tiles = cdiv(kv_len, kTileRows);
+  plan.summary_bytes = tile_summary_bytes(batch, kv_len);
+  if (want_wide && head_dim == 128) {  // lists of live tiles per 256 query rows, shared by the heads
+    const size_t bytes = tile_list_bytes(batch, q_len, kWideTileRows, kv_len);
+    if (bytes > 0 && bytes <= kMaxTileListBytes && live_tiles_bytes(8, n_kv_tiles) <= kLdsPerCu) {
+      plan.wide = true;
+      plan.list_bytes = bytes;
+    }
+  }
   const int64_t regular = (int64_t)batch * num_heads * cdiv(q_len, kSplitTileRows);
   // the ring of the four-wavefront configuration (see launch_fwd_auto) and its share of the LDS
   const int ring_bytes = (2 * kTK * head_dim * 2 + 2 * kTK * 4) * (head_dim == 64 ? 3 : 2);
   if (ring_bytes + live_tiles_bytes(4, n_kv_tiles) > (head_dim == 256 ? kLdsPerCu : kLdsHalfCu)) return plan;
   if (q_len >= kSplitTileRows && regular >= 256) return plan;
   plan.split_mode = true;
+  plan.list_bytes = 0;
+  plan.wide = false;
   const int64_t rows = (int64_t)q_len * (num_heads / num_kv_heads);
   const int64_t items = (int64_t)batch * num_kv_heads * ((rows + kSplitTileRows - 1) / kSplitTileRows);
   // windows of one size for every item, at most 64 per item
@@ -588,6 +976,7 @@ FwdPlan plan_forward(int batch, int q_len, int kv_len, int num_heads, int num_kv
     plan.part_o_bytes = (slots * head_dim * sizeof(float) + 15) / 16 * 16;
     plan.part_ml_bytes = (slots * 2 * sizeof(float) + 15) / 16 * 16;
   }
+  if (plan.narrow()) plan.summary_bytes = 0;
   return plan;
 }
 
@@ -624,6 +1013,21 @@ int launch_fwd(const FwdParams& p0, hipStream_t stream) {
   return KVAX_OK;
 }
 
+template <class Tr, int D>
+int launch_fwd_wide(const FwdParams& p0, hipStream_t stream) {
+  FwdParams p = p0;
+  p.num_splits = p.num_parts = 1;
+  p.num_q_tiles = cdiv(p.q_len, kWideTileRows);
+  p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_q_tiles, p.group}.grid();
+  if (p.batch * p.num_heads * p.num_q_tiles == 0) return KVAX_OK;
+  auto kernel = fa_fwd_wide_kernel<Tr, D>;
+  constexpr int smem = FwdSmem<D, 2>::kTotal;
+  static LdsReservation reservation;
+  if (int rc = reservation.ensure(kernel, kLdsPerCu, "the wide forward kernel")) return rc;
+  hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(256), smem, stream, p);
+  return check_launch("fa_fwd_wide_kernel");
+}
+
 // Two work-groups of four wavefronts per compute unit (each hides the other's prologue, barriers
 // and final stores) whenever the tile bitmaps of the sequence fit beside the smaller ring;
 // otherwise one work-group of eight wavefronts.
@@ -658,7 +1062,8 @@ int validate_fa_common(const kvax_fa_args* a) {
     return fail(KVAX_EUNSUPPORTED, "head_dim %d is not built (64, 128 and 256 are)", a->head_dim);
   if (a->dtype != KVAX_BF16 && a->dtype != KVAX_F16)
     return fail(KVAX_EUNSUPPORTED, "dtype %d is not supported (bf16 and f16 are)", a->dtype);
-  if (a->flags & ~(KVAX_FA_DKDV_F32 | KVAX_FA_SKIP_DELTA | KVAX_FA_SKIP_DQ | KVAX_FA_SKIP_DKDV)) return fail(KVAX_EINVAL, "unknown bits in flags");
+  if (a->flags & ~(KVAX_FA_DKDV_F32 | KVAX_FA_SKIP_DELTA | KVAX_FA_SKIP_DQ | KVAX_FA_SKIP_DKDV | KVAX_FA_FWD_WIDE))
+    return fail(KVAX_EINVAL, "unknown bits in flags");
   // empty tensors may come with null pointers
   const bool has_q = a->batch > 0 && a->q_len > 0, has_kv = a->batch > 0 && a->kv_len > 0;
   if ((has_q && (!a->q || !a->out || !a->lse || !a->q_pos || !a->q_seg)) ||
@@ -683,9 +1088,9 @@ using namespace kvax;
 
 extern "C" size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* a) {
   if (!a || a->batch < 0 || a->kv_len < 0) return 0;
-  // kv tile summaries, then the partial results of the split mode
-  const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim);
-  return tile_summary_bytes(a->batch, a->kv_len) + plan.part_o_bytes + plan.part_ml_bytes;
+  // see FwdPlan
+  return plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim,
+                                    (a->flags & KVAX_FA_FWD_WIDE) != 0).total_bytes();
 }
 
 // Scratch memory of kvax_fa_fwd_static: one copy per GPU the library runs on, held until the
@@ -716,7 +1121,7 @@ int static_scratch(void** ptr) {
   return KVAX_OK;
 }
 
-int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, kvax_stream_t stream_);
+int fa_fwd_impl(const kvax_fa_args* a, void* workspace, kvax_stream_t stream_);
 
 }  // namespace
 
@@ -726,7 +1131,7 @@ extern "C" int kvax_fa_fwd(const kvax_fa_args* a, void* workspace, size_t worksp
   const size_t need = kvax_fa_fwd_workspace_bytes(a);
   if (need > workspace_bytes || (need && !workspace))
     return fail(KVAX_EWORKSPACE, "workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-  return fa_fwd_impl(a, workspace, workspace_bytes, stream_);
+  return fa_fwd_impl(a, workspace, stream_);
 }
 
 extern "C" int kvax_fa_fwd_static(const kvax_fa_args* a, kvax_stream_t stream_) {
@@ -738,14 +1143,13 @@ extern "C" int kvax_fa_fwd_static(const kvax_fa_args* a, kvax_stream_t stream_) 
                 kStaticScratchBytes);
   void* ws = nullptr;
   if (int rc = static_scratch(&ws)) return rc;
-  // Nothing in the buffer has to start at zero: the tile summaries and, in split mode, every
-  // partial result that is read are written by this call's own kernels first.
-  return fa_fwd_impl(a, ws, kStaticScratchBytes, stream_);
+  // Nothing in the buffer has to start at zero: the tile summaries, the lists and, in split mode,
+  // every partial result that is read are written by this call's own kernels first.
+  return fa_fwd_impl(a, ws, stream_);
 }
 
 namespace {
-int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, kvax_stream_t stream_) {
-  (void)workspace_bytes;
+int fa_fwd_impl(const kvax_fa_args* a, void* workspace, kvax_stream_t stream_) {
   if ((uintptr_t)workspace % 16) return fail(KVAX_EINVAL, "workspace must be 16-byte aligned");
   if (a->fwd_query_block <= 0 || a->fwd_kv_block <= 0)
     return fail(KVAX_EINVAL, "forward block sizes must be positive");
@@ -779,29 +1183,38 @@ int fa_fwd_impl(const kvax_fa_args* a, void* workspace, size_t workspace_bytes, 
   p.scale_log2 = fmaxf(fabsf(a->scale), 1e-30f) * 1.4426950408889634f;
   p.kv_tiles = (const int4*)workspace;
   p.n_kv_tiles = cdiv(a->kv_len, kTileRows);
-  {
-    const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim);
-    p.split_mode = plan.split_mode;
-    p.num_splits = plan.num_splits;
-    p.num_parts = plan.num_parts;
-    p.split_tiles = plan.split_tiles;
-    p.part_rows = plan.part_rows;
-    p.part_o = (float*)((char*)workspace + tile_summary_bytes(a->batch, a->kv_len));
-    p.part_ml = (float*)((char*)p.part_o + plan.part_o_bytes);
-  }
+  const FwdPlan plan = plan_forward(a->batch, a->q_len, a->kv_len, a->num_heads, a->num_kv_heads, a->head_dim,
+                                    (a->flags & KVAX_FA_FWD_WIDE) != 0);
+  p.split_mode = plan.split_mode;
+  p.num_splits = plan.num_splits;
+  p.num_parts = plan.num_parts;
+  p.split_tiles = plan.split_tiles;
+  p.part_rows = plan.part_rows;
+  p.part_o = (float*)((char*)workspace + plan.summary_bytes);
+  p.part_ml = (float*)((char*)p.part_o + plan.part_o_bytes);
+  uint32_t* lists = plan.wide ? (uint32_t*)((char*)p.part_ml + plan.part_ml_bytes) : nullptr;
+  p.lists = lists;
+  p.list_stride = (int)tile_list_stride(p.n_kv_tiles);
   hipStream_t stream = (hipStream_t)stream_;
-  if (a->q_len == 0 || a->batch == 0) return KVAX_OK;
-  {  // too long for the largest configuration: refuse before anything is enqueued
+  if (!plan.wide) {  // too long for the largest configuration: refuse before anything is enqueued
     const int ring = (2 * kTK * a->head_dim * 2 + 2 * kTK * 4) * (a->head_dim == 256 ? 2 : 3);
     const int need = ring + live_tiles_bytes(a->head_dim == 256 ? 4 : 8, p.n_kv_tiles);
     if (need > kLdsPerCu)
       return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)",
                   a->kv_len, need, kLdsPerCu);
   }
-  if (!(p.split_mode && p.num_parts > p.num_splits)) {  // the narrow mode does not read them
+  if (!plan.narrow()) {  // the narrow mode does not read them
     TileSummaryJob job{a->kv_pos, a->kv_seg, workspace, a->kv_len};
     if (int rc = launch_tile_summaries(&job, 1, a->batch, stream)) return rc;
   }
+  if (lists) {
+    TileListJob job{a->q_pos, a->q_seg, {a->fwd_mask[0], a->fwd_mask[1], a->fwd_mask[2], a->fwd_mask[3]},
+                    workspace, lists, a->q_len, a->kv_len, a->fwd_query_block, a->fwd_kv_block,
+                    p.n_qblocks, p.n_kv_tiles, kWideTileRows / 32};
+    if (int rc = launch_tile_lists(job, a->batch, stream)) return rc;
+  }
+  if (plan.wide)
+    return a->dtype == KVAX_BF16 ? launch_fwd_wide<Bf16, 128>(p, stream) : launch_fwd_wide<F16, 128>(p, stream);
   const bool bf16 = a->dtype == KVAX_BF16;
   if (a->head_dim == 256)
     return bf16 ? launch_fwd_auto<Bf16, 256>(p, stream) : launch_fwd_auto<F16, 256>(p, stream);

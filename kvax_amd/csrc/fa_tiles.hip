@@ -132,7 +132,84 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
   }
 }
 
+// See TileListJob.  One work-group per (item, batch row) with the item's wavefronts, each taking the 32
+// rows it owns in the attention kernels.
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void tile_lists_kernel(TileListJob job) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+  const int item = blockIdx.x, b = blockIdx.y;
+  constexpr int kRows = NW * 32;
+  const int q0 = item * kRows;
+  // range of the item: union of [lower, upper) over its mask blocks, intersection of the full ranges
+  int lo = 0x7fffffff, hi = 0, flo = 0, fhi = 0x7fffffff;
+  {
+    const int qb0 = q0 / job.qbs, qb1 = min((q0 + kRows - 1) / job.qbs, job.n_qblocks - 1);
+    for (int qb = qb0; qb <= qb1; qb++) {
+      const int64_t mi = (int64_t)b * job.n_qblocks + qb;
+      const int l_ = job.mask[0][mi] * job.kbs, u_ = job.mask[1][mi] * job.kbs;
+      flo = max(flo, job.mask[2][mi] * job.kbs);
+      fhi = min(fhi, job.mask[3][mi] * job.kbs);
+      if (u_ > l_) {
+        lo = min(lo, l_);
+        hi = max(hi, u_);
+      }
+    }
+  }
+  hi = min(hi, job.kv_len);
+  const int t_lo = lo / kTileRows;
+  const int t_hi = hi > lo ? (hi + kTileRows - 1) / kTileRows : t_lo;
+  const int tf_lo = (flo + kTileRows - 1) / kTileRows, tf_hi = fhi / kTileRows;
+
+  // the wavefront's rows (both half-waves hold the same 32)
+  const int row = q0 + wave * 32 + lane % 32;
+  const bool in = row < job.q_len;
+  const int qi = in ? row : 0;
+  const int seg = job.q_seg[(int64_t)b * job.q_len + qi], pos = job.q_pos[(int64_t)b * job.q_len + qi];
+  const int64_t mi = (int64_t)b * job.n_qblocks + qi / job.qbs;
+  const int col_lo = job.mask[0][mi] * job.kbs;
+  const int col_width = max(min(job.mask[1][mi] * job.kbs, job.kv_len) - col_lo, 0);
+  const int4* kv_summaries = reinterpret_cast<const int4*>(job.kv_tiles) + 2 * (int64_t)b * job.n_kv_tiles;
+  const WordSummaries first_word = load_word_summaries(kv_summaries, t_lo >> 6, t_lo, t_hi, lane);
+  TileParts mine[1];
+  mine[0] = wave_parts(in && seg != -1 && col_width > 0, seg, pos);
+
+  int* live_count = reinterpret_cast<int*>(smem);
+  unsigned long long* live_bits = reinterpret_cast<unsigned long long*>(smem + 16);
+  const int word0 = t_lo >> 6;
+  const int words = t_hi > t_lo ? ((t_hi - 1) >> 6) - word0 + 1 : 0;
+  uint32_t* live_list = reinterpret_cast<uint32_t*>(live_bits + NW * (cdiv_dev(job.n_kv_tiles, 64) + 1));
+  mark_live_tiles<true, 1>(kv_summaries, mine, t_lo, t_hi, live_bits + wave * words, word0, lane, first_word);
+  __syncthreads();
+  if (wave == 0) compact_live_tiles<NW>(live_bits, words, word0, live_list, live_count, lane);
+  __syncthreads();
+  const int n = *live_count;
+  uint32_t* out = job.lists + ((size_t)b * gridDim.x + item) * tile_list_stride(job.n_kv_tiles);
+  if (threadIdx.x == 0)
+    *reinterpret_cast<uint4*>(out) = make_uint4((uint32_t)n, (uint32_t)tf_lo, (uint32_t)tf_hi, 0u);
+  for (int j = threadIdx.x; j < n; j += NW * 64) out[4 + j] = live_list[j];
+}
+
 }  // namespace
+
+int launch_tile_lists(const TileListJob& job, int batch, hipStream_t stream) {
+  if (job.waves != 4 && job.waves != 8) return fail(KVAX_EINVAL, "tile lists for items of %d wavefronts", job.waves);
+  const int items = cdiv(job.q_len, job.waves * 32);
+  if (items == 0 || batch == 0) return KVAX_OK;
+  const int smem = live_tiles_bytes(job.waves, job.n_kv_tiles);
+  if (smem > kLdsPerCu)
+    return fail(KVAX_EUNSUPPORTED, "kv_len %d needs %d bytes of LDS for tile bitmaps (limit %d)", job.kv_len, smem, kLdsPerCu);
+  if (job.waves == 4) {
+    static LdsReservation reservation;
+    if (int rc = reservation.ensure(tile_lists_kernel<4>, kLdsPerCu, "the tile list kernel")) return rc;
+    hipLaunchKernelGGL(tile_lists_kernel<4>, dim3(items, batch), dim3(256), smem, stream, job);
+  } else {
+    static LdsReservation reservation;
+    if (int rc = reservation.ensure(tile_lists_kernel<8>, kLdsPerCu, "the tile list kernel")) return rc;
+    hipLaunchKernelGGL(tile_lists_kernel<8>, dim3(items, batch), dim3(512), smem, stream, job);
+  }
+  return check_launch("tile_lists_kernel");
+}
 
 int launch_tile_order(const TileOrderJob& job, int batch, hipStream_t stream) {
   if (job.sub < 1 || job.sub > 4) return fail(KVAX_EINVAL, "work items of %d tiles", job.sub);

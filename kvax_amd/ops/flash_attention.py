@@ -106,11 +106,12 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
 
 
 def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd_mask, scale,
-                            fwd_params, bwd_params, buffers=None, static_scratch=False):
+                            fwd_params, bwd_params, buffers=None, static_scratch=False, flags=0):
     """One device's forward: returns (out like query, lse fp32 [batch, heads, q_len]).
     ``buffers`` = (out, lse) lets a caller reuse its output tensors.  With ``static_scratch`` (and
     ``buffers``) the call goes through ``kvax_fa_fwd_static`` and allocates no device memory: the
-    scratch memory is the library's own fixed buffer, shared by all calls on the GPU."""
+    scratch memory is the library's own fixed buffer, shared by all calls on the GPU.  ``flags``:
+    ``_native.KVAX_FA_FWD_WIDE`` selects the kernel variant with 64 query rows per wavefront."""
     b, sq, hq, d = query.shape
     if buffers is not None:
         out, lse = buffers
@@ -120,6 +121,7 @@ def flash_attention_forward(query, key, value, q_pos, q_seg, kv_pos, kv_seg, fwd
     a = _base_args(query, key, value, q_pos, q_seg, kv_pos, kv_seg, scale, fwd_params, bwd_params)
     a.out, a.lse, a.o_strides = out.data_ptr(), lse.data_ptr(), _strides3(out)
     a.fwd_mask = _mask_ptrs(fwd_mask)
+    a.flags = flags
     lib = _native.lib()
     if static_scratch:
         with torch.cuda.device(query.device):

@@ -197,30 +197,39 @@ def test_constant_positions_are_bidirectional(device):
 _HEADS_ORACLE = {}
 
 
-def _sampled_heads_oracle(name, heads):
-    """Oracle output of a few heads of a full-size workload (batch row 0), computed once per
+def _sampled_heads_oracle(name, heads, row=0):
+    """Oracle output of a few heads of one batch row of a full-size workload, computed once per
     process: it does not depend on the mask block size."""
-    if name not in _HEADS_ORACLE:
+    key = (name, tuple(heads), row)
+    if key not in _HEADS_ORACLE:
         w = workload(name)
         q, k, v = w.draw_tensors(0, "cpu", with_dout=False)
-        ref, _ = ao.attention_forward(q[:1].float().numpy(), k[:1].float().numpy(), v[:1].float().numpy(),
-                                      w.q_pos[:1], w.q_seg[:1], w.kv_pos[:1], w.kv_seg[:1],
+        r = slice(row, row + 1)
+        ref, _ = ao.attention_forward(q[r].float().numpy(), k[r].float().numpy(), v[r].float().numpy(),
+                                      w.q_pos[r], w.q_seg[r], w.kv_pos[r], w.kv_seg[r],
                                       w.scale, dtype=np.float32, heads=heads, row_block=2048)
-        _HEADS_ORACLE[name] = ref
-    return _HEADS_ORACLE[name]
+        _HEADS_ORACLE[key] = ref
+    return _HEADS_ORACLE[key]
 
 
-@pytest.mark.parametrize("name, block, heads", [("dense_causal", 128, [0, 13]), ("doc32k", 128, [5]),
-                                                ("block_skip", 128, [0, 63]), ("block_skip", 64, [0, 63])])
-def test_measurement_workloads_sampled_heads(device, name, block, heads):
+# heads from different kv groups; for the four-row block_skip workload also the last batch row (its
+# byte offsets are the largest of all configurations)
+@pytest.mark.parametrize("name, block, heads, row", [
+    ("dense_causal", 128, [0, 13], 0), ("doc32k", 128, [5, 26], 0),
+    ("block_skip", 128, [0, 63], 0), ("block_skip", 64, [0, 63], 0),
+    ("block_skip", 128, [0, 63], 3), ("block_skip", 64, [0, 63], 3)])
+def test_measurement_workloads_sampled_heads(device, name, block, heads, row):
     """Full-size configurations at every mask block size they are specified for; the dense oracle is
-    evaluated for a sample of heads of the first batch row."""
+    evaluated for a sample of heads of one batch row."""
     w = workload(name, block=block)
     q, k, v = w.draw_tensors(0, device, with_dout=False)
     data = (q, k, v) + w.ids(device)
     assert w.fwd_blocks == (block, block)
     out = run_forward(data, w.scale, *w.fwd_blocks)
-    check(out[:1], _sampled_heads_oracle(name, heads), data[4][:1], heads=heads)
+    r = slice(row, row + 1)
+    err = np.abs(out[r].float().cpu().numpy()[:, :, heads] - _sampled_heads_oracle(name, heads, row)[:, :, heads]).max()
+    print(f"{name} block {block} row {row} heads {heads}: max abs err {err:.3e}")
+    check(out[r], _sampled_heads_oracle(name, heads, row), data[4][r], heads=heads)
 
 
 def test_unsorted_document_ids(device):
@@ -357,3 +366,78 @@ def test_randomized_short_query_shapes(device, seed):
     data, scale, block = _short_query_case(seed)
     out = run_forward(tuple(x.to(device) for x in data), scale, block, block)
     check(out, oracle_forward(data, scale), data[4])
+
+
+@pytest.mark.parametrize("sq, qbs", [(1, 1), (64, 32)])
+def test_split_mode_padding_queries_with_masks_that_keep_padding(device, sq, qbs):
+    """Split mode with masks built with ``skip_pad_tokens=False``, which declare blocks of padding
+    queries against padding keys mask-free: work-groups whose rows are all padding (an inactive slot
+    of a decoding batch: the narrow path; the padded half of a chunk of 64 new tokens: windows with
+    live-tile lists) accumulate over those blocks without the element mask and must still write
+    exact zeros."""
+    sk, hq, hkv, batch = 4096, 8, 2, 3
+    g = torch.Generator().manual_seed(sq)
+    q = torch.randn((batch, sq, hq, 128), generator=g).to(torch.bfloat16).to(device)
+    k = torch.randn((batch, sk, hkv, 128), generator=g).to(torch.bfloat16).to(device)
+    v = torch.randn((batch, sk, hkv, 128), generator=g).to(torch.bfloat16).to(device)
+    filled = sk - 1500  # key cache: `filled` tokens, then padding
+    kv_pos = torch.arange(sk, dtype=torch.int32)[None].repeat(batch, 1)
+    kv_seg = torch.zeros((batch, sk), dtype=torch.int32)
+    kv_seg[:, filled:] = -1
+    q_pos = kv_pos[:, filled - sq:filled].clone()
+    q_seg = torch.zeros((batch, sq), dtype=torch.int32)
+    if sq == 1:  # batch row 1 is an inactive slot
+        q_seg[1, :], q_pos[1, :] = -1, sk + 10
+    else:        # the second half of every chunk is padding
+        q_seg[:, sq // 2:], q_pos[:, sq // 2:] = -1, sk + 10
+    ids = tuple(x.to(device) for x in (q_pos, q_seg, kv_pos, kv_seg))
+    params = FlashAttentionParamsConfig(qbs, 128)
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(*ids, fwd_params=params, skip_pad_tokens=False)
+        out = flash_attention(q, k, v, *ids, mask, scale=128 ** -0.5, fwd_params=params)
+    # the case is the intended one: some query block sees the padding keys as a mask-free range
+    m = mask[0]
+    assert ((m.upper_full_bounds - m.lower_full_bounds) * 128 >= 1024).any()
+    data = (q, k, v) + ids
+    check(out, oracle_forward(data, 128 ** -0.5), ids[1])
+
+
+def _forward_with_flags(data, scale, block, flags):
+    from kvax_amd import _native
+    from kvax_amd.ops.flash_attention import flash_attention_forward
+    q, k, v, *ids = data
+    params = FlashAttentionParamsConfig(block, block)
+    with attention_specs(*TP_SPECS):
+        mask = create_attention_mask(*ids, fwd_params=params)
+    out, lse = flash_attention_forward(q, k, v, *ids, mask[0], scale, params, params,
+                                       flags=_native.KVAX_FA_FWD_WIDE if flags else 0)
+    return out, lse
+
+
+@pytest.mark.parametrize("sq, sk, hq, hkv, pad, nseg, block", [
+    (2048, 2048, 8, 2, 77, 5, 128),     # documents and padding
+    (2000, 1900, 8, 8, 0, 1, 64),       # ragged lengths, one document
+    (4096, 4096, 4, 1, 600, 12, 128),   # many documents, multi-query
+])
+def test_wide_forward_kernel(device, sq, sk, hq, hkv, pad, nseg, block):
+    """KVAX_FA_FWD_WIDE (64 query rows per wavefront, one wavefront per SIMD) against the oracle and
+    against the default kernel (same values up to the rounding of a different summation order)."""
+    lengths = generate_random_segments_lengths(min(sq, sk), nseg)
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, 128, 128, seed=sq + nseg,
+                                               num_pad_tokens=pad, list_of_segment_lengths=lengths,
+                                               device=device)
+    wide, lse_w = _forward_with_flags(data, scale, block, True)
+    plain, lse_p = _forward_with_flags(data, scale, block, False)
+    check(wide, oracle_forward(data, scale), data[4])
+    assert (wide.float() - plain.float()).abs().max().item() <= 1.6e-2
+    assert (lse_w - lse_p).abs().max().item() <= 1e-3
+
+
+def test_wide_forward_kernel_restarting_positions(device):
+    """The wide kernel on the 32k document workload (positions restart per document, padding tail):
+    two heads against the dense oracle."""
+    w = workload("doc32k")
+    q, k, v = w.draw_tensors(0, device, with_dout=False)
+    data = (q, k, v) + w.ids(device)
+    out, _ = _forward_with_flags(data, w.scale, 128, True)
+    check(out[:1], _sampled_heads_oracle("doc32k", [5, 26]), data[4][:1], heads=[5, 26])

@@ -196,15 +196,25 @@ def test_workspace_sizes_follow_the_shapes():
     bwd = lambda *s: lib.kvax_fa_bwd_workspace_bytes(ctypes.byref(_fa_args(*s)))
     assert fwd(1, 32768, 32768, 32, 8, 128) == 32 * 512                 # training shape: summaries only
     assert fwd(4, 8192, 8192, 16, 16, 128) == 4 * 32 * 128
-    summaries = 8 * 32 * 512
-    decode = fwd(8, 1, 32768, 32, 8, 128)                               # one query per row: split mode
-    assert decode > summaries
-    partial_bytes = decode - summaries
+    # one query per row: split mode with at most 32 rows per kv head, which walks every tile of its
+    # windows and needs no summaries - partial results only
+    partial_bytes = fwd(8, 1, 32768, 32, 8, 128)
+    assert partial_bytes > 0
+    # 40 queries per row (160 rows per kv head): split mode with live-tile lists - summaries as well
+    assert fwd(8, 40, 32768, 32, 8, 128) > 8 * 32 * 512
     # 64 work items (8 rows x 8 kv heads) x windows x 4 rows x (128 + 2) floats, 16-byte aligned pieces
     assert partial_bytes % (64 * 4 * 4) == 0
     windows = partial_bytes // (64 * 4 * (128 + 2) * 4)
     assert 2 <= windows <= 64 and windows * 64 * 4 * 130 * 4 == partial_bytes
     assert fwd(8, 1, 64, 32, 8, 128) == 8 * 32                          # too short to divide
+    # the wide forward variant adds one list of live tiles (4 header words + one per kv tile) per 256
+    # query rows; the request is ignored where the variant does not apply
+    wide = _fa_args(1, 32768, 32768, 32, 8, 128)
+    wide.flags = _native.KVAX_FA_FWD_WIDE
+    assert lib.kvax_fa_fwd_workspace_bytes(ctypes.byref(wide)) == 32 * 512 + 128 * (4 + 512) * 4
+    wide = _fa_args(1, 32768, 32768, 32, 8, 64)
+    wide.flags = _native.KVAX_FA_FWD_WIDE
+    assert lib.kvax_fa_fwd_workspace_bytes(ctypes.byref(wide)) == 32 * 512
     assert fwd(0, 1, 32768, 32, 8, 128) == 0
     delta = 1 * 32 * 32768 * 4
     order = (2 * 256 + 1) * 4 + 12                                      # 256 kv work items, padded to 16
