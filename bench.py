@@ -4,12 +4,16 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload doc32k]
 
 A step is one forward + backward pass of document-mask attention over one batch of seeded
-synthetic tensors that already live in HBM, through the C ABI (kvax_fa_fwd, kvax_fa_bwd).  The
+synthetic tensors that already live in HBM, through the C ABI (one kvax_fa_fwd and one kvax_fa_bwd
+call, as a training step issues them).  The per-kernel times come from a second, untimed pass that
+runs the backward's two kernels in separate calls with HIP events around each.  The
 block masks are built once before the loop, as a training step would build them once per batch
 and reuse them across layers; their build time is reported separately (``mask_build_ms``).
 After the headline workload (doc32k) the other configurations of the baseline - dense causal forward,
 the context-parallel shard, the block-skipping case at mask blocks 128 and 64, and a decoding step -
 are timed for a few steps each and reported under ``other_workloads`` of the same line.
+A library bf16 GEMM is timed in the same run (``mfma_reference``): what this machine's matrix
+pipeline sustains for plain GEMMs, with the shader clock read while it runs.
 Prints ONE JSON line.  ``value`` counts only unmasked FLOPs: 4*D per attendable (q, kv) pair
 and query head in the forward, 2.5x that in the backward.
 """
@@ -77,6 +81,11 @@ def parse():
                     help="also run a plain streaming kernel of known size (reads and writes "
                          f"{CALIBRATION_BYTES >> 20} MiB) so that a rocprofv3 --pmc run of this command "
                          "shows what FETCH_SIZE / WRITE_SIZE read for a known amount of HBM traffic")
+    ap.add_argument("--fwd-wide", action="store_true",
+                    help="run the forward with KVAX_FA_FWD_WIDE (64 query rows per wavefront, one wavefront "
+                         "per SIMD): a variant kept to measure what halving the LDS traffic buys")
+    ap.add_argument("--no-mfma-reference", action="store_true",
+                    help="skip the library GEMM timed for the mfma_reference object")
     ap.add_argument("--global-positions", action="store_true",
                     help="positions = token index instead of restarting per document")
     return ap.parse_args()
@@ -117,6 +126,33 @@ def sample_sclk(step, ms_per_step, seconds=0.4, samples=8):
             got.append(v)
     torch.cuda.synchronize()
     return (float(np.mean(got)), len(got)) if got else None
+
+
+def mfma_reference(n=8192, iters=20):
+    """What the matrix pipeline of this machine sustains for a plain library GEMM: torch.matmul of two
+    n x n bf16 matrices (hipBLASLt), `iters` calls timed with HIP events after a warm-up, and the shader
+    clock the driver reports while the same GEMMs run again.  The attention kernels cannot be faster
+    per MFMA than this: they do their element-wise work on top."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    a = torch.randn((n, n), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    b = torch.randn((n, n), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    c = torch.empty((n, n), device=dev, dtype=torch.bfloat16)
+    for _ in range(5):
+        torch.matmul(a, b, out=c)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        torch.matmul(a, b, out=c)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / iters
+    tflops = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+    sclk = sample_sclk(lambda: torch.matmul(a, b, out=c), ms)
+    return {"what": f"torch.matmul, bf16, {n} x {n} x {n}, {iters} calls", "value": tflops, "unit": "TFLOP/s",
+            "ms": ms, "frac_of_datasheet_peak": tflops / MFMA_BF16_DENSE_PEAK_TFLOPS,
+            "clock_under_load_mhz": sclk[0] if sclk else None}
 
 
 def cpu_baseline(w, seed, seconds_hint=20.0):
@@ -198,6 +234,24 @@ def measure(args, name, block, steps, warmup, device_tensors=False):
         m1.record()
         torch.cuda.synchronize()
         mask_ms = m0.elapsed_time(m1) / reps
+        # the same calls without the host in the way: `reps` of them captured in one HIP graph (kernels
+        # only, no memset nodes) and replayed, which leaves the device time of a call's two kernels
+        mask_gpu_ms = None
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                for _ in range(reps):
+                    create_attention_mask(*ids, fwd_params=fp, bwd_params=bp, calc_bwd_mask=True)
+            graph.replay()
+            torch.cuda.synchronize()
+            m0.record()
+            graph.replay()
+            m1.record()
+            torch.cuda.synchronize()
+            mask_gpu_ms = m0.elapsed_time(m1) / reps
+            del graph
+        except RuntimeError:
+            mask_gpu_ms = None
 
     # ---- reusable outputs / workspace ----------------------------------------------------------
     out = torch.empty_like(q)
@@ -206,37 +260,45 @@ def measure(args, name, block, steps, warmup, device_tensors=False):
     ws = torch.empty(backward_workspace_bytes(q, k) + 16, dtype=torch.uint8, device=dev)
     SQ, SK = _native.KVAX_FA_SKIP_DQ, _native.KVAX_FA_SKIP_DKDV
 
+    fwd_flags = _native.KVAX_FA_FWD_WIDE if args.fwd_wide else 0
+
     def fwd():
-        flash_attention_forward(q, k, v, *ids, masks[0], w.scale, fp, bp, buffers=(out, lse))
+        flash_attention_forward(q, k, v, *ids, masks[0], w.scale, fp, bp, buffers=(out, lse), flags=fwd_flags)
 
     def bwd(flags):
         flash_attention_backward(q, k, v, *ids, masks[1], masks[2], out, lse, dout, w.scale, fp, bp,
                                  flags=flags, buffers=(dq, dk, dv, ws))
 
+    # the timed step: one forward call and one backward call
+    def step():
+        fwd()
+        if backward:
+            bwd(0)
+
+    # per-kernel pass (untimed for `value`): the backward's kernels in separate calls
     phases = [("fa_fwd_kernel", fwd)]
     if backward:
         # the dQ kernel also produces delta = rowsum(O * dO), which the dK/dV kernel reads
         phases += [("fa_bwd_dq_kernel", lambda: bwd(SK)),
                    ("fa_bwd_dkdv_kernel", lambda: bwd(SQ))]
 
-    def step(events=None):
-        for i, (_, fn) in enumerate(phases):
-            if events is not None:
-                events[i][0].record()
-            fn()
-            if events is not None:
-                events[i][1].record()
-
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    all_events = [[(ev(), ev()) for _ in phases] for _ in range(steps)]
     t0 = time.perf_counter()
     for s_ in range(steps):
-        step(all_events[s_])
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / steps
+
+    all_events = [[(ev(), ev()) for _ in phases] for _ in range(steps)]
+    for s_ in range(steps):
+        for i, (_, fn) in enumerate(phases):
+            all_events[s_][i][0].record()
+            fn()
+            all_events[s_][i][1].record()
+    torch.cuda.synchronize()
     kernel_ms = {name_: float(np.mean([all_events[s_][i][0].elapsed_time(all_events[s_][i][1])
                                        for s_ in range(steps)]))
                  for i, (name_, _) in enumerate(phases)}
@@ -268,7 +330,7 @@ def measure(args, name, block, steps, warmup, device_tensors=False):
     figures = {
         "sclk": sclk,
         "value": value, "ms_per_step": ms_per_step, "pairs": pairs, "f_step": f_step, "f_fwd": f_fwd,
-        "roofline": roofline, "mask_build_ms": mask_ms, "kernel_ms": kernel_ms,
+        "roofline": roofline, "mask_build_ms": mask_ms, "mask_build_gpu_ms": mask_gpu_ms, "kernel_ms": kernel_ms,
         "kernel_tflops": {n: (kernel_flops[n] / (ms * 1e-3) / 1e12 if ms > 0 else 0.0)
                           for n, ms in kernel_ms.items()},
     }
@@ -331,11 +393,16 @@ def main():
             "flops_per_step": m["f_step"],
             "num_documents": len(w.meta.get("doc_lengths", [])) or None,
             "padding_tokens": w.meta.get("pad"),
+            "forward_kernel": "wide (KVAX_FA_FWD_WIDE)" if args.fwd_wide else "default",
         },
         "roofline": m["roofline"],
         "step_frac_of_mfma_peak": m["value"] / MFMA_BF16_DENSE_PEAK_TFLOPS,
         "fwd_tflops": m["f_fwd"] / (m["kernel_ms"]["fa_fwd_kernel"] * 1e-3) / 1e12,
+        # create_attention_mask(calc_bwd_mask=True): per call as the host sees it (20 calls back to
+        # back), and the device time per call (the 20 calls replayed from one HIP graph)
         "mask_build_ms": m["mask_build_ms"],
+        "mask_build_gpu_ms": m["mask_build_gpu_ms"],
+        # per-kernel times: a separate pass with the backward's two kernels in separate calls
         "kernel_ms": m["kernel_ms"],
         "kernel_tflops": m["kernel_tflops"],
         # the peak above assumes the datasheet's 2.4 GHz; this is the shader clock the driver reported
@@ -355,10 +422,18 @@ def main():
                 "value_is": "forward+backward TFLOP/s" if w2.backward else "forward TFLOP/s",
                 "ms_per_step": m2["ms_per_step"], "unmasked_pairs": m2["pairs"],
                 "roofline": m2["roofline"], "mask_build_ms": m2["mask_build_ms"],
+                "mask_build_gpu_ms": m2["mask_build_gpu_ms"],
                 "kernel_ms": m2["kernel_ms"], "kernel_tflops": m2["kernel_tflops"],
             }
             del w2, m2
         result["other_workloads"] = others
+    if not args.no_mfma_reference:
+        torch.cuda.empty_cache()
+        ref = mfma_reference()
+        result["mfma_reference"] = ref
+        if result["roofline"]["bound"] == "mfma":
+            result["roofline"]["frac_of_reference"] = result["roofline"]["achieved"] / ref["value"]
+            result["step_frac_of_mfma_reference"] = result["value"] / ref["value"]
     if not args.no_cpu_baseline:
         from kvax_amd.utils.benchmarking import workload
         result["cpu_baseline"] = cpu_baseline(workload(args.workload, seed=args.seed,

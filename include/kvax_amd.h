@@ -165,6 +165,9 @@ int kvax_fa_bwd(const kvax_fa_args* args, void* workspace, size_t workspace_byte
  * kvax_fa_fwd_workspace_bytes() exceeds that size fails with KVAX_EWORKSPACE and enqueues nothing
  * (long key sequences in split mode are the only such case: 8 MiB cover 32 rows x 32 query heads
  * decoding against 128k keys).  The call allocates and frees nothing and does not synchronise.
+ * The first call of each kernel variant (head_dim, dtype, regular / split / decoding shape class) on
+ * a device makes the HIP runtime load that kernel and look up the scratch buffer's address: make one
+ * call per variant outside stream capture first, as for any kernel that is to be captured.
  * All calls on one GPU share the buffer: calls that overlap in time on one GPU (different streams
  * or host threads) race; serialise them or use kvax_fa_fwd with separate workspaces. */
 #define KVAX_FA_FWD_STATIC_MAX_WORKSPACE (8u << 20)

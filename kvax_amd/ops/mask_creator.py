@@ -31,7 +31,36 @@ def _as_ids(x: DeviceArray, name: str) -> torch.Tensor:
         raise _native.KvaxNativeError(
             f"{name} lives on {x.device}: the mask builder only runs on the GPU"
         )
+    if x.dtype is torch.int32 and x.is_contiguous():
+        return x
     return x.to(torch.int32).contiguous()
+
+
+_LAYOUTS: dict = {}
+
+
+def _layout(lib, batch, q_len, kv_len, requests, num_q_shards):
+    """Where the masks of a call lie in its one allocation (in int32 words after the workspace), and
+    the workspace size; a function of the shapes and block sizes, remembered per distinct call."""
+    key = (batch, q_len, kv_len, requests, num_q_shards)
+    hit = _LAYOUTS.get(key)
+    if hit is not None:
+        return hit
+    descs = (_native.MaskDesc * len(requests))()
+    shapes = []
+    words = 0
+    for d, (qbs, kbs, kv_outer) in zip(descs, requests):
+        n_outer = -(-kv_len // kbs) if kv_outer else -(-q_len // qbs)
+        shards = num_q_shards if kv_outer else 1
+        d.query_block_size, d.kv_block_size, d.kv_outer = qbs, kbs, int(kv_outer)
+        shapes.append((words, batch, shards, n_outer))
+        words += (4 * batch * shards * n_outer + 3) // 4 * 4  # masks start on 16-byte boundaries
+    ws_bytes = lib.kvax_mask_workspace_bytes(batch, q_len, kv_len, descs, len(requests))
+    ws_words = (max(ws_bytes, 16) + 15) // 16 * 4
+    if len(_LAYOUTS) > 256:
+        _LAYOUTS.clear()
+    _LAYOUTS[key] = (shapes, words, ws_bytes, ws_words)
+    return _LAYOUTS[key]
 
 
 def build_masks(
@@ -43,7 +72,11 @@ def build_masks(
     skip_pad_tokens: bool = True,
     num_q_shards: int = 1,
 ) -> list[AttentionMask]:
-    """Build one mask per ``(query_block_size, kv_block_size, kv_outer)`` request in one call."""
+    """Build one mask per ``(query_block_size, kv_block_size, kv_outer)`` request in one call.
+
+    The host side of a call is kept short (it is most of the call's latency: the two kernels take
+    under 10 us): one device allocation holds the workspace and every mask, whose tensors are views
+    of it."""
     if not 1 <= len(requests) <= _native.KVAX_MAX_MASKS:
         raise ValueError(f"between 1 and {_native.KVAX_MAX_MASKS} masks per call")
     q_pos = _as_ids(query_positions, "query_positions")
@@ -56,28 +89,39 @@ def build_masks(
         raise ValueError("query and kv batch sizes differ")
     batch, q_len = q_pos.shape
     kv_len = kv_pos.shape[1]
+    device = q_pos.device
     lib = _native.lib()
     descs = (_native.MaskDesc * len(requests))()
-    outs = []
+    layout = _layout(lib, batch, q_len, kv_len, tuple(requests), num_q_shards)
+    shapes, words, ws_bytes, ws_words = layout
     for d, (qbs, kbs, kv_outer) in zip(descs, requests):
-        n_outer = -(-kv_len // kbs) if kv_outer else -(-q_len // qbs)
-        shards = num_q_shards if kv_outer else 1
-        buf = torch.empty((4, batch, shards, n_outer), dtype=torch.int32, device=q_pos.device)
         d.query_block_size, d.kv_block_size, d.kv_outer = qbs, kbs, int(kv_outer)
-        d.lower, d.upper = buf[0].data_ptr(), buf[1].data_ptr()
-        d.lower_full, d.upper_full = buf[2].data_ptr(), buf[3].data_ptr()
-        outs.append(buf)
-    ws_bytes = lib.kvax_mask_workspace_bytes(batch, q_len, kv_len, descs, len(requests))
-    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q_pos.device)
-    stream = torch.cuda.current_stream(q_pos.device).cuda_stream
-    with torch.cuda.device(q_pos.device):
+    buf = torch.empty(ws_words + words, dtype=torch.int32, device=device)
+    base = buf.data_ptr()
+    masks = []
+    for d, (off, b, shards, n_outer) in zip(descs, shapes):
+        n = b * shards * n_outer
+        first = base + 4 * (ws_words + off)
+        d.lower, d.upper, d.lower_full, d.upper_full = first, first + 4 * n, first + 8 * n, first + 12 * n
+        views = buf[ws_words + off:ws_words + off + 4 * n].view(4, b, shards, n_outer).unbind(0)
+        masks.append(AttentionMask(*views))
+    stream = torch.cuda.current_stream(device).cuda_stream
+    index = device.index
+    if index is None or index == torch.cuda.current_device():
         rc = lib.kvax_mask_build(
             q_pos.data_ptr(), q_seg.data_ptr(), kv_pos.data_ptr(), kv_seg.data_ptr(),
             batch, q_len, kv_len, num_q_shards, int(skip_pad_tokens),
-            descs, len(requests), ws.data_ptr(), ws_bytes, C.c_void_p(stream),
+            descs, len(requests), base, ws_bytes, C.c_void_p(stream),
         )
+    else:
+        with torch.cuda.device(device):
+            rc = lib.kvax_mask_build(
+                q_pos.data_ptr(), q_seg.data_ptr(), kv_pos.data_ptr(), kv_seg.data_ptr(),
+                batch, q_len, kv_len, num_q_shards, int(skip_pad_tokens),
+                descs, len(requests), base, ws_bytes, C.c_void_p(stream),
+            )
     _native.check(rc, "kvax_mask_build")
-    return [AttentionMask(b[0], b[1], b[2], b[3]) for b in outs]
+    return masks
 
 
 def compute_attention_mask(

@@ -93,9 +93,10 @@ def test_sequential_positions_equal_explicit_arange(device):
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("rank", [0, 3, 7])
-def test_cp_shard_workload_against_oracle(device, rank):
-    """One CP=8 shard of a 131072-token sequence at real shape; oracle on one GQA group."""
+@pytest.mark.parametrize("rank, group", [(0, 1), (3, 1), (7, 1), (3, 6)])
+def test_cp_shard_workload_against_oracle(device, rank, group):
+    """One CP=8 shard of a 131072-token sequence at real shape; oracle on one GQA group (kv head
+    `group`: query heads 4 * group ... 4 * group + 3)."""
     w = workload("cp_shard", cp_rank=rank)
     q, k, v, dout = w.draw_tensors(0, device, with_dout=True)
     ids = w.ids(device)
@@ -107,7 +108,7 @@ def test_cp_shard_workload_against_oracle(device, rank):
         assert tuple(masks[2].lower_bounds.shape) == (1, 1, 1024)
         out = flash_attention(q, k, v, *ids, masks, scale=w.scale, fwd_params=fp, bwd_params=bp)
     out.backward(dout)
-    heads = [4, 5, 6, 7]
+    heads = [4 * group + i for i in range(4)]
     f = lambda t: t.detach().float().cpu().numpy()
     args = (f(q), f(k), f(v), w.q_pos, w.q_seg, w.kv_pos, w.kv_seg, w.scale)
     ref_out, _ = ao.attention_forward(*args, dtype=np.float32, heads=heads, row_block=1024)
@@ -115,16 +116,16 @@ def test_cp_shard_workload_against_oracle(device, rank):
     # 2e-2 plus the rounding of the 16-bit result (tests/tolerances.py)
     worst = {"out": check_close("out", out[:, :, heads], ref_out[:, :, heads]),
              "dq": check_close("dq", q.grad[:, :, heads], ref_dq[:, :, heads]),
-             "dk": check_close("dk", k.grad[:, :, 1], ref_dk[:, :, 1]),
-             "dv": check_close("dv", v.grad[:, :, 1], ref_dv[:, :, 1])}
+             "dk": check_close("dk", k.grad[:, :, group], ref_dk[:, :, group]),
+             "dv": check_close("dv", v.grad[:, :, group], ref_dv[:, :, group])}
     # dK/dV of the sampled kv head straight from the fp32 accumulators: plain 2e-2
     with torch.no_grad():
         out2, lse = flash_attention_forward(q, k, v, *ids, masks[0], w.scale, fp, bp)
         _, dk32, dv32 = flash_attention_backward(q, k, v, *ids, masks[1], masks[2], out2, lse, dout,
                                                  w.scale, fp, bp, dkdv_fp32=True)
-    worst["dk fp32"] = check_close("dk fp32", dk32[:, :, 1], ref_dk[:, :, 1])
-    worst["dv fp32"] = check_close("dv fp32", dv32[:, :, 1], ref_dv[:, :, 1])
-    print(f"  cp_shard rank {rank}: " + ", ".join(f"{n} {e:.3e}" for n, e in worst.items()))
+    worst["dk fp32"] = check_close("dk fp32", dk32[:, :, group], ref_dk[:, :, group])
+    worst["dv fp32"] = check_close("dv fp32", dv32[:, :, group], ref_dv[:, :, group])
+    print(f"  cp_shard rank {rank} group {group}: " + ", ".join(f"{n} {e:.3e}" for n, e in worst.items()))
 
 
 @pytest.mark.parametrize("heads, kv_heads, batch", [(6, 3, 1), (4, 2, 1), (2, 1, 1), (8, 8, 3)])

@@ -314,6 +314,27 @@ def test_split_mode_matches_dense_oracle(device, sq, sk, hq, hkv, d, batch, pad,
     check(out, oracle_forward(data, scale), data[4])
 
 
+@pytest.mark.parametrize("sq, hq, hkv, d", [(1, 16, 4, 128), (24, 8, 2, 64)])
+def test_split_mode_fp16(device, sq, hq, hkv, d):
+    """fp16 through the split mode: one query per row (the narrow decoding path, 4 rows per kv head)
+    and a chunk of 24 new tokens (96 rows per kv head: windows with live-tile lists), with documents
+    over the key cache."""
+    sk = 6000
+    data, scale = make_random_attention_inputs(2, sq, sk, hq, hkv, d, d, seed=sq + d, num_pad_tokens=0,
+                                               start_query_position=sk - sq, dtype=torch.float16,
+                                               device=device)
+    q, k, v, q_pos, q_seg, kv_pos, kv_seg = data
+    assert q.dtype == torch.float16
+    bounds = np.cumsum([0, 1500, 2500, 2000])
+    seg_of = torch.from_numpy(np.searchsorted(bounds, np.arange(sk), side="right") - 1).to(torch.int32).to(device)
+    kv_seg = seg_of[None].expand_as(kv_seg).contiguous()
+    q_seg = seg_of[q_pos.clamp(max=sk - 1).long()]
+    data = (q, k, v, q_pos, q_seg, kv_pos, kv_seg)
+    out = run_forward(data, scale, 128, 128)
+    assert out.dtype == torch.float16
+    check(out, oracle_forward(data, scale), q_seg)
+
+
 def test_decode_workload_all_rows(device):
     """The decode measurement workload (one query per row, key caches filled to different lengths)
     against the oracle, every batch row and head."""

@@ -29,12 +29,20 @@ def bound(ref: np.ndarray, dtype, atol: float = ATOL) -> np.ndarray:
     return atol + half_ulp(np.abs(ref) + atol, dtype)
 
 
-def check_close(name: str, got: torch.Tensor, ref: np.ndarray, atol: float = ATOL) -> float:
-    """Asserts |got - ref| <= bound(ref, got.dtype) everywhere; returns the largest error."""
+# P and dS enter the second contractions rounded to the 16-bit input dtype (as the reference
+# prescribes, flash_attention_triton.py:128,513,610): each product carries a relative error of up to
+# 2^-9.  On gradients that sum eight or more query heads into one kv head and reach |dK|, |dV| of
+# 10-20 this alone is 1-2.5e-2 (measured), whatever the accumulators do; the fp32 checks of those
+# cases add this relative term to the 2e-2.
+OPERAND_ROUNDING = 2.0 ** -10
+
+
+def check_close(name: str, got: torch.Tensor, ref: np.ndarray, atol: float = ATOL, rel: float = 0.0) -> float:
+    """Asserts |got - ref| <= bound(ref, got.dtype) + rel * |ref| everywhere; returns the largest error."""
     g = got.detach().float().cpu().numpy()
     assert np.isfinite(g).all(), f"{name}: non-finite values"
     err = np.abs(g - ref)
-    worst = (err - bound(ref, got.dtype, atol)).max() if err.size else 0.0
+    worst = (err - bound(ref, got.dtype, atol) - rel * np.abs(ref)).max() if err.size else 0.0
     top = float(err.max()) if err.size else 0.0
     assert worst <= 0, (f"{name} ({got.dtype}): max abs err {top:.4g} exceeds {atol:g} + half ulp "
                         f"(|ref| max {np.abs(ref).max():.3g}, excess {worst:.3g})")
