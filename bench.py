@@ -50,6 +50,7 @@ def recorded_traffic(kernel: str, workload_name: str):
 
 WORKLOAD_TEXT = {
     "dense_causal": "dense_causal: B1 S8192 Hq32/Hkv8 D128 bf16, one causal document, block 128, forward only",
+    "dense64k": "dense64k: B1 S65536 Hq4/Hkv1 D128 bf16, one causal document, block 128, forward only",
     "doc32k": "doc32k: B1 S32768 Hq32/Hkv8 D128 bf16, causal document mask, lognormal document "
               "lengths (median 2048, sigma 1, clip [128,16384]), ~5% trailing padding, positions "
               "restart per document, dO~N(0,1), block 128, forward+backward",

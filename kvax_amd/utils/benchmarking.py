@@ -233,6 +233,9 @@ def workload(name: str, seed: int = 0, restart_positions: bool = True, cp_rank: 
 
     ``cpu_plumbing``   B1 S2048 Hq8/Hkv2 D64 fp32, 4 documents + 128 padding tokens, causal, block 64
     ``dense_causal``   B1 S8192 32/8 D128 bf16, one document, forward only, block 128
+    ``dense64k``       B1 S65536 4/1 D128 bf16, one document, forward only, block 128: the same FLOPs
+                       per head as 64 heads at 16k, in few long rows (the loops of the forward kernel
+                       with almost nothing else: used to compare kernel variants)
     ``doc32k``         B1 S32768 32/8 D128 bf16, lognormal documents (median 2048, sigma 1,
                        clipped to [128, 16384]) + ~5 % padding, forward + backward, block 128
     ``cp_shard``       queries = chunks (r, 15-r) of a 131072-token sequence cut in 16, keys =
@@ -255,6 +258,12 @@ def workload(name: str, seed: int = 0, restart_positions: bool = True, cp_rank: 
         S = 8192
         pos, seg = _layout_documents([S], S, restart_positions)
         return Workload(name, 1, S, S, 32, 8, 128, True, (128, 128), (128, 128), False,
+                        pos[None], seg[None], pos[None].copy(), seg[None].copy(),
+                        meta=dict(seed=seed, doc_lengths=[S], pad=0))
+    if name == "dense64k":
+        S = 65536
+        pos, seg = _layout_documents([S], S, restart_positions)
+        return Workload(name, 1, S, S, 4, 1, 128, True, (128, 128), (128, 128), False,
                         pos[None], seg[None], pos[None].copy(), seg[None].copy(),
                         meta=dict(seed=seed, doc_lengths=[S], pad=0))
     if name == "doc32k":

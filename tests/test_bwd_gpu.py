@@ -65,7 +65,7 @@ def fp32_dkdv(data, scale, fwd_blocks, bwd_blocks, dout):
 
 def check_fp32_dkdv(data, scale, fwd_blocks, bwd_blocks, dout, refs):
     """Where the 16-bit dK/dV get the relaxed 5e-2 (one kv head summing 8 or more query heads, as
-    the reference relaxes it), the fp32 results are held to 2e-2 + 2^-10 |ref|: the rounding of P
+    the reference relaxes it), the fp32 results are held to 2e-2 + 2^-10 max |ref|: the rounding of P
     and dS to the input dtype, which the accumulators cannot undo (see tests/tolerances.py; the
     largest errors seen are 2.6e-2 at |dV| = 18.5 and 2.2e-2 at |dK| = 8.3)."""
     dk, dv = fp32_dkdv(data, scale, fwd_blocks, bwd_blocks, dout)

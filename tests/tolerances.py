@@ -38,11 +38,14 @@ OPERAND_ROUNDING = 2.0 ** -10
 
 
 def check_close(name: str, got: torch.Tensor, ref: np.ndarray, atol: float = ATOL, rel: float = 0.0) -> float:
-    """Asserts |got - ref| <= bound(ref, got.dtype) + rel * |ref| everywhere; returns the largest error."""
+    """Asserts |got - ref| <= bound(ref, got.dtype) + rel * max |ref| everywhere (the rounding of the
+    operands of a sum scales with the terms summed, not with the sum's own value); returns the
+    largest error."""
     g = got.detach().float().cpu().numpy()
     assert np.isfinite(g).all(), f"{name}: non-finite values"
     err = np.abs(g - ref)
-    worst = (err - bound(ref, got.dtype, atol) - rel * np.abs(ref)).max() if err.size else 0.0
+    scale = float(np.abs(ref).max()) if err.size else 0.0
+    worst = (err - bound(ref, got.dtype, atol) - rel * scale).max() if err.size else 0.0
     top = float(err.max()) if err.size else 0.0
     assert worst <= 0, (f"{name} ({got.dtype}): max abs err {top:.4g} exceeds {atol:g} + half ulp "
                         f"(|ref| max {np.abs(ref).max():.3g}, excess {worst:.3g})")
