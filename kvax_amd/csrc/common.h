@@ -76,8 +76,9 @@ inline size_t tile_summary_bytes(int batch, int len) {
 // rows and writes the tiles that are live for at least one wavefront, in ascending order:
 //   list[0] = number of entries, list[1], list[2] = first tile and end of the mask-free tile range,
 //   list[4 + j] = tile index | (mask of the wavefronts it is live for) << 24
-// (what every work-group of the attention kernels would otherwise work out for itself - the same
-// list for each of the query heads).  Lists are `tile_list_stride(n_kv_tiles)` words apart.
+// (the same list serves every query head of the batch row).  Only the wide forward kernel reads these
+// lists; the other attention kernels work theirs out in LDS per work-group, which measured the same.
+// Lists are `tile_list_stride(n_kv_tiles)` words apart.
 struct TileListJob {
   const int32_t* q_pos;
   const int32_t* q_seg;
@@ -94,8 +95,8 @@ __host__ __device__ inline size_t tile_list_stride(int n_kv_tiles) { return (siz
 inline size_t tile_list_bytes(int batch, int q_len, int rows_per_item, int kv_len) {
   return (size_t)batch * cdiv(q_len, rows_per_item) * tile_list_stride(cdiv(kv_len, kTileRows)) * sizeof(uint32_t);
 }
-// Above this size the lists are not built and the attention kernels fall back to working them out in
-// LDS per work-group (the size grows with q_len * kv_len / 8192 * 4 bytes: 0.5 MB for 32k x 32k).
+// Above this size the lists are not built and a call that asks for the wide forward kernel runs the
+// default one (the size grows with q_len * kv_len / 16384 * 4 bytes: 0.26 MB for 32k x 32k).
 #ifndef KVAX_MAX_TILE_LIST_MB
 #define KVAX_MAX_TILE_LIST_MB 64
 #endif
