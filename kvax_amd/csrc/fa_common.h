@@ -126,7 +126,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 // L % 8, each XCD has its own L2), so the map from L to a work item decides both L2 sharing and
 // balance.  Items are (group, tile rank, member): a group is one (batch, kv head) -- everything
 // that reads the same K/V -- with `tiles` tiles ranked heaviest first and `members` query heads
-// per tile.  With at least 8 groups each XCD owns whole groups; with fewer (and 8 divisible by
+// per tile.  With at least 8 groups each XCD owns whole groups (visited in an order that rotates
+// from rank to rank, see decode()); with fewer (and 8 divisible by
 // the count) the tiles of a group are dealt round-robin to the XCDs that share it, so that every
 // XCD gets the same mix of heavy and light tiles; otherwise items are cut into 8 contiguous runs.
 struct ItemMap {
@@ -142,9 +143,17 @@ struct ItemMap {
     const int x = L % 8, j = L / 8;
     if (mode() == 0) {
       const int per_xcd = (groups + 7) / 8;
+      const int jm = j / members;
       member = j % members;
-      group = x + 8 * ((j / members) % per_xcd);
-      rank = j / (members * per_xcd);
+      rank = jm / per_xcd;
+      // The work-groups of an XCD go to its four shader engines in turn (work-group j to engine
+      // j % 4, measured), and an engine that is full holds back the ones behind it.  With a number
+      // of items per rank that shares a factor with 4, an engine would get the same groups (batch
+      // rows) at every rank, and rows differ in work: the groups are rotated from rank to rank so
+      // that every engine sees all of them.
+      const int per_rank = per_xcd * members;
+      const int every = per_rank % 4 == 0 ? 1 : (per_rank % 2 == 0 ? 2 : 4);  // 4 / gcd(per_rank, 4)
+      group = x + 8 * ((jm + rank / every) % per_xcd);
       return group < groups && rank < tiles;
     }
     if (mode() == 1) {
