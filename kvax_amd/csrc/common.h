@@ -62,7 +62,9 @@ struct TileSummaryJob {
   void* out;  // int4 [batch, cdiv(len, kTileRows), 2]
   int len;
 };
-// `zero` (optional): `batch` int32 counters the kernel clears, for a following launch_tile_order().
+// `zero` (optional): `batch` + kQueueCounters int32 counters the kernel clears: the arrival counters
+// of a following launch_tile_order() and the item queues of the dK/dV kernel (one per XCD).
+constexpr int kQueueCounters = 8;
 int launch_tile_summaries(const TileSummaryJob* jobs, int num_jobs, int batch, hipStream_t stream,
                           int32_t* zero = nullptr);
 inline size_t tile_summary_bytes(int batch, int len) {
@@ -106,10 +108,12 @@ constexpr size_t kMaxTileListBytes = (size_t)KVAX_MAX_TILE_LIST_MB << 20;
 // work-group owns); its work is the number of tiles of the other sequence that at least one of its
 // tiles can interact with according to the summaries.  Writes, per batch row, the dispatch order of
 // the items: those with more than the row's mean work in index order, then the others by decreasing
-// work (ties: lower index first), so that the launch ends on short items.  One launch; `ws` holds
-// the order (the result, int32 [batch, n_items], at the start), then the work counts and one
-// arrival counter per batch row, which launch_tile_summaries() must have zeroed (pass it
-// tile_order_counters(ws, ...)).
+// work (ties: lower index first), so that the launch ends on short items; entries of items whose
+// work is zero carry the flag kDeadItem.  One launch; `ws` holds
+// the order (the result, int32 [batch, n_items], at the start), then the work counts, one
+// arrival counter per batch row and kQueueCounters item counters for the kernel that consumes the
+// order, all of which launch_tile_summaries() must have zeroed (pass it tile_order_counters(ws, ...)).
+constexpr int kDeadItem = 1 << 30;  // flag on an entry of the order: the item's work count is zero
 struct TileOrderJob {
   const void* own;   // summaries of the items' sequence, int4 [batch, n_own, 2]
   const void* opp;   // summaries of the streamed sequence, int4 [batch, n_opp, 2]
@@ -119,7 +123,7 @@ struct TileOrderJob {
 };
 int launch_tile_order(const TileOrderJob& job, int batch, hipStream_t stream);
 inline size_t tile_order_bytes(int batch, int n_items) {
-  return ((size_t)batch * (2 * n_items + 1) * sizeof(int32_t) + 15) / 16 * 16;
+  return (((size_t)batch * (2 * n_items + 1) + kQueueCounters) * sizeof(int32_t) + 15) / 16 * 16;
 }
 inline int32_t* tile_order_counters(int32_t* ws, int batch, int n_items) {
   return ws + (size_t)batch * 2 * n_items;

@@ -62,6 +62,7 @@ struct BwdParams {
   int list_tiles;  // dK/dV kernel: query tiles per chunk of the live-tile bookkeeping
   int32_t* order_ws;           // room for the dK/dV dispatch order and its scratch
   const int32_t* dkdv_order;   // dispatch order of the kv tiles [batch, tiles], or null
+  int32_t* dkdv_queue;         // dK/dV kernel: one item counter per XCD, zero at launch
   int flags;
   float scale, scale_log2;
   float scale_log2_abs;  // |scale| * log2(e) > 0, used with K negated when the scale is negative
@@ -424,15 +425,56 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   const int pair = wave % NP;
   const bool p_wave = wave < NP;  // role, wave-uniform
 
+  // The launch is one work-group per compute unit, and each takes work items (128 kv rows of one
+  // batch row and kv head) from the queue of its XCD until none is left: item j of XCD x is what
+  // work-group 8 j + x of a launch with one work-group per item would be.  (The hardware deals the
+  // work-groups of a launch to an XCD's four shader engines in strict rotation and in order, so a
+  // compute unit that finishes a long work-group waits until the rotation comes round to its
+  // engine: measured 6 to 12 % of this kernel's compute-unit time idle between work-groups.)  The
+  // index of the next item is requested when the current one's step loop has ended, so that its
+  // latency hides behind the final stores and an item is never held back by a long one.  A
+  // work-group whose XCD has run out of items takes them from the other XCDs' queues (the XCDs do
+  // not run at exactly the same speed): that costs L2 sharing, but only at the end of the launch.
+  const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, 1};
+  int queue = blockIdx.x % 8;  // the queue this work-group currently draws from (thread 0 only)
+  // thread 0: the launch-wide index of the item that `ticket` of the current queue stands for, moving
+  // on to the next queue while the current one is exhausted; -1 when all are
+  auto resolve = [&](int ticket) {
+    for (int tries = 0;; tries++) {
+      const int id = 8 * ticket + queue;
+      if (id < p.total_items) return id;
+      if (tries == 7) return -1;
+      queue = (queue + 1) % 8;
+      ticket = atomicAdd(p.dkdv_queue + queue, 1);
+    }
+  };
+  int* next_item = reinterpret_cast<int*>(smem + Smem::kTotal) + 1;
+  if (tid == 0) *next_item = resolve(atomicAdd(p.dkdv_queue + queue, 1));
+  __syncthreads();
+  for (int item = *next_item; item >= 0; item = *next_item) {
+  __syncthreads();  // every wavefront has read next_item
+  int ticket = 0;
   // kv tiles in the computed dispatch order (without one: early tiles first, which see the most
   // queries under a causal mask)
   int group, rank, member;
-  const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, 1};
-  if (!items.decode(blockIdx.x, group, rank, member)) return;
+  if (items.decode(item, group, rank, member)) {
   const int kv_head = group % p.num_kv_heads;
   const int b = group / p.num_kv_heads;
-  const int kv_tile = p.dkdv_order ? p.dkdv_order[(int64_t)b * p.num_tiles + rank] : rank;
+  const int entry = p.dkdv_order ? p.dkdv_order[(int64_t)b * p.num_tiles + rank] : rank;
+  const int kv_tile = entry & (kDeadItem - 1);
   const int k0 = kv_tile * TKV;
+  if (entry & kDeadItem) {
+    // no query tile can interact with these kv rows (known from the ordering pass): zeros, no bookkeeping
+    if (tid == 0) ticket = atomicAdd(p.dkdv_queue + queue, 1);
+    const int row_bytes = D * (p.dkdv_f32 ? 4 : 2), chunks = row_bytes / 16;
+    const int rows = min(TKV, p.kv_len - k0);
+    for (int i = tid; i < rows * chunks; i += NW * 64) {
+      const int64_t row = k0 + i / chunks;
+      const int at = (i % chunks) * 16;
+      *reinterpret_cast<uint4*>(p.dk + ((int64_t)b * p.dk_sb + (int64_t)kv_head * p.dk_sh + row * p.dk_ss) * (row_bytes / D) + at) = make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4*>(p.dv + ((int64_t)b * p.dv_sb + (int64_t)kv_head * p.dv_sh + row * p.dv_ss) * (row_bytes / D) + at) = make_uint4(0, 0, 0, 0);
+    }
+  } else {
 
   const int kbs = p.bk, qbs = p.bq;
   const int64_t mbase = (int64_t)b * p.n_kv_blocks;
@@ -738,37 +780,71 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   __syncthreads();  // the next chunk reuses the bookkeeping, the rings and the exchange slots
   }
 
+  if (tid == 0) ticket = atomicAdd(p.dkdv_queue + queue, 1);
   // ---- epilogue: the P wave holds dV^T, the S wave dK^T (times the scale) ----------------------
-  if (in) {
+  // A lane holds 4 consecutive head-dim elements of its kv row per register group, so storing from
+  // the registers would touch 32 rows with 8 or 16 bytes each per instruction.  Each wavefront
+  // instead passes its 32 x D tile through its own part of the LDS (the rings are free by now),
+  // 128 head-dim columns at a time, and writes whole rows: 16 bytes per lane, consecutive lanes
+  // consecutive chunks of a row.  Rows are swizzled by the row index so that neither side has bank
+  // conflicts.
+  {
     const bool dead = col_width == 0;  // padding keys: exact zeros (see the dQ kernel's epilogue)
     const float mul = p_wave ? 1.f : p.scale;
     char* base = p_wave ? p.dv : p.dk;
     const int64_t sb = p_wave ? p.dv_sb : p.dk_sb, sh = p_wave ? p.dv_sh : p.dk_sh, ss = p_wave ? p.dv_ss : p.dk_ss;
-    const int64_t off = (int64_t)b * sb + (int64_t)kv_head * sh + (int64_t)kvcol * ss;
-    if (p.dkdv_f32) {
-      float* row = reinterpret_cast<float*>(base) + off;
+    constexpr int PC = D < 128 ? D : 128;  // columns per pass
+    constexpr int kDtPerPass = PC / 32;
+    const int esize = p.dkdv_f32 ? 4 : 2;
+    const int row_bytes = PC * esize;             // 128, 256 or 512
+    const int chunks = row_bytes / 16;            // 8, 16 or 32 per row
+    char* stage = smem + wave * (32 * PC * 4);    // room for the fp32 case
+    const int64_t tile_off = (int64_t)b * sb + (int64_t)kv_head * sh + (int64_t)(k0 + pair * 32) * ss;
 #pragma unroll
-      for (int dt = 0; dt < DT; dt++)
+    for (int pass = 0; pass < D / PC; pass++) {
+      char* mine = stage + c * row_bytes;
+      if (p.dkdv_f32) {
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++)
-          *reinterpret_cast<float4*>(row + 32 * dt + 8 * g4 + 4 * h) =
-              dead ? make_float4(0.f, 0.f, 0.f, 0.f)
-                   : make_float4(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul,
-                                 acc[dt][4 * g4 + 2] * mul, acc[dt][4 * g4 + 3] * mul);
-    } else {
-      char* row = base + off * 2;
+        for (int d = 0; d < kDtPerPass; d++)
 #pragma unroll
-      for (int dt = 0; dt < DT; dt++)
+          for (int g4 = 0; g4 < 4; g4++) {
+            const f32x16& a = acc[pass * kDtPerPass + d];
+            const int chunk = 8 * d + 2 * g4 + h;
+            *reinterpret_cast<float4*>(mine + ((chunk ^ (c & (chunks - 1))) * 16)) =
+                dead ? make_float4(0.f, 0.f, 0.f, 0.f)
+                     : make_float4(a[4 * g4 + 0] * mul, a[4 * g4 + 1] * mul, a[4 * g4 + 2] * mul, a[4 * g4 + 3] * mul);
+          }
+      } else {
 #pragma unroll
-        for (int g4 = 0; g4 < 4; g4++) {
-          uint2 u;
-          u.x = Tr::pack2(acc[dt][4 * g4 + 0] * mul, acc[dt][4 * g4 + 1] * mul);
-          u.y = Tr::pack2(acc[dt][4 * g4 + 2] * mul, acc[dt][4 * g4 + 3] * mul);
-          if (dead) u = make_uint2(0, 0);
-          *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
-        }
+        for (int d = 0; d < kDtPerPass; d++)
+#pragma unroll
+          for (int g4 = 0; g4 < 4; g4++) {
+            const f32x16& a = acc[pass * kDtPerPass + d];
+            uint2 u;
+            u.x = Tr::pack2(a[4 * g4 + 0] * mul, a[4 * g4 + 1] * mul);
+            u.y = Tr::pack2(a[4 * g4 + 2] * mul, a[4 * g4 + 3] * mul);
+            if (dead) u = make_uint2(0, 0);
+            const int chunk = 4 * d + g4;
+            *reinterpret_cast<uint2*>(mine + ((chunk ^ (c & (chunks - 1))) * 16) + 8 * h) = u;
+          }
+      }
+      // 32 rows x `chunks` 16-byte pieces, 64 per instruction
+      const int per_iter = 64 / chunks;  // rows per instruction: 8, 4 or 2
+      for (int r0 = 0; r0 < 32; r0 += per_iter) {
+        const int row = r0 + lane / chunks, chunk = lane % chunks;
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + row * row_bytes + ((chunk ^ (row & (chunks - 1))) * 16));
+        if (k0 + pair * 32 + row < p.kv_len)
+          *reinterpret_cast<uint4*>(base + (tile_off + (int64_t)row * ss) * esize + pass * row_bytes + chunk * 16) = v;
+      }
     }
   }
+  }  // the item has work
+  } else if (tid == 0) {
+    ticket = atomicAdd(p.dkdv_queue + queue, 1);
+  }
+  if (tid == 0) *next_item = resolve(ticket);
+  __syncthreads();
+  }  // items of this XCD
 }
 
 template <class K>
@@ -857,7 +933,8 @@ int launch_bwd(BwdParams p, hipStream_t stream) {
     if (int rc = reserve_lds(kernel, smem, kLdsLimit, &done, "the dK/dV kernel")) return rc;
     p.num_tiles = cdiv(p.kv_len, Cfg::kKvRows);
     p.total_items = ItemMap{p.batch * p.num_kv_heads, p.num_tiles, 1}.grid();
-    hipLaunchKernelGGL(kernel, dim3(p.total_items), dim3(NW * 64), smem, stream, p);
+    p.dkdv_queue = tile_order_counters(p.order_ws, p.batch, p.num_tiles) + p.batch;
+    hipLaunchKernelGGL(kernel, dim3(min(p.total_items, kNumCus)), dim3(NW * 64), smem, stream, p);
     if (int rc = check_launch("fa_bwd_dkdv_kernel")) return rc;
   }
   return KVAX_OK;

@@ -16,13 +16,16 @@ namespace {
 
 struct Params {
   TileSummaryJob jobs[2];
-  int32_t* zero;  // one counter per batch row to clear, or null
+  int32_t* zero;  // counters to clear (one per batch row, then kQueueCounters more), or null
 };
 
 __global__ __launch_bounds__(256) void tile_summaries_kernel(Params p) {
   const TileSummaryJob& job = p.jobs[blockIdx.z];
   const int lane = threadIdx.x % 64;
-  if (p.zero && blockIdx.x == 0 && blockIdx.z == 0 && threadIdx.x == 0) p.zero[blockIdx.y] = 0;
+  if (p.zero && blockIdx.x == 0 && blockIdx.z == 0) {
+    if (threadIdx.x == 0) p.zero[blockIdx.y] = 0;
+    if (blockIdx.y == 0 && threadIdx.x < kQueueCounters) p.zero[gridDim.y + threadIdx.x] = 0;
+  }
   const int n_tiles = (job.len + kTileRows - 1) / kTileRows;
   const int tile = blockIdx.x * 4 + threadIdx.x / 64;
   if (tile >= n_tiles) return;
@@ -128,7 +131,8 @@ __global__ __launch_bounds__(256) void tile_order_kernel(TileOrderJob job, int b
       const int4 k = *reinterpret_cast<const int4*>(keys + j);
       rank += (k.x < mine) + (k.y < mine) + (k.z < mine) + (k.w < mine);
     }
-    order[rank] = i;
+    // an item without any work (it ranks among the last) is marked, so that its consumer need not find out
+    order[rank] = mine == job.n_items * (1 + job.n_opp) + i ? i | kDeadItem : i;
   }
 }
 
