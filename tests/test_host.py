@@ -190,7 +190,7 @@ def test_workspace_sizes_follow_the_shapes():
     """The workspace functions are pure functions of the shapes (no GPU needed): 32 bytes per
     64-row tile and batch row for the summaries; the forward adds room for partial results only
     where it runs in its split mode (short query sequences); the backward holds delta, both
-    summaries and the dispatch order of the dK/dV work items."""
+    summaries, the order of the dK/dV work items and the counters of their queues."""
     lib = _native.lib()
     fwd = lambda *s: lib.kvax_fa_fwd_workspace_bytes(ctypes.byref(_fa_args(*s)))
     bwd = lambda *s: lib.kvax_fa_bwd_workspace_bytes(ctypes.byref(_fa_args(*s)))
@@ -217,7 +217,7 @@ def test_workspace_sizes_follow_the_shapes():
     assert lib.kvax_fa_fwd_workspace_bytes(ctypes.byref(wide)) == 32 * 512
     assert fwd(0, 1, 32768, 32, 8, 128) == 0
     delta = 1 * 32 * 32768 * 4
-    order = (2 * 256 + 1) * 4 + 12                                      # 256 kv work items, padded to 16
+    order = (2 * 256 + 1 + 8) * 4 + 12      # 256 kv work items, an arrival counter, 8 queue counters; padded to 16
     assert bwd(1, 32768, 32768, 32, 8, 128) == delta + 2 * 32 * 512 + order
 
 
