@@ -142,6 +142,20 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
   const int t_hi = r.hi > r.lo ? (r.hi + kTile - 1) / kTile : t_lo;
   const int tf_lo = (r.flo + kTile - 1) / kTile, tf_hi = r.fhi / kTile;
 
+  if (t_hi <= t_lo) {
+    // No row of the tile can attend to anything (padding queries): zeros for dQ and delta, and
+    // nothing is read.  Whole rows, 16 bytes per lane.
+    constexpr int kChunks = D * 2 / 16;
+    const int rows = min(TQ, p.q_len - q0);
+    char* dq0 = p.dq + ((int64_t)b * p.dq_sb + (int64_t)head * p.dq_sh) * 2;
+    for (int i = tid; i < rows * kChunks; i += NW * 64)
+      *reinterpret_cast<uint4*>(dq0 + (int64_t)(q0 + i / kChunks) * p.dq_ss * 2 + (i % kChunks) * 16) =
+          make_uint4(0, 0, 0, 0);
+    for (int i = tid; i < rows; i += NW * 64)
+      p.delta[((int64_t)b * p.num_heads + head) * p.q_len + q0 + i] = 0.f;
+    return;
+  }
+
   // per-lane query column.  Its ids, its row of the block mask and lse are read without waiting
   // for one another (index 0 stands in for rows beyond the sequence), as are dO, O, Q and the first
   // 64 tile summaries below: one trip to memory for the whole prologue instead of several in a row.

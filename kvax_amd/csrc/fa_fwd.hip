@@ -175,6 +175,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   }
   const int tf_lo = (flo + kTK - 1) / kTK, tf_hi = fhi / kTK;
 
+  if (!SPLIT && t_hi <= t_lo) {
+    // No row of the tile can attend to anything (padding queries): zeros for O and lse, and nothing
+    // is read.  Whole rows, 16 bytes per lane.
+    constexpr int kChunks = D * 2 / 16;
+    const int rows = min(TQ, p.q_len - q0);
+    for (int i = tid; i < rows * kChunks; i += NW * 64)
+      *reinterpret_cast<uint4*>(obase + (int64_t)(q0 + i / kChunks) * p.o_ss * 2 + (i % kChunks) * 16) =
+          make_uint4(0, 0, 0, 0);
+    for (int i = tid; i < rows; i += NW * 64) lse[q0 + i] = 0.f;
+    return;
+  }
+
   // ---- per-lane query columns ------------------------------------------------------------
   // qrow: the lane's query index; lane_head: its query head (split mode: per lane).
   // Everything the prologue reads from memory that does not depend on another read - the lane's
