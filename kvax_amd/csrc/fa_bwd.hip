@@ -349,12 +349,18 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
     }
   }
 
-  if (in) {
+  {
     // Rows that attend to nothing (padding) get exact zeros.  Their accumulator is not zero when the
     // block mask declares padding-against-padding blocks mask-free (masks built without skipping
     // padding): the element mask, which is what excludes them, is not applied there.
+    // The rows leave through LDS (each wavefront its own part of the tile space, which is done with)
+    // as whole rows, 16 bytes per lane, instead of 8-byte pieces of 32 rows per store; rows are
+    // swizzled by the row index against bank conflicts.
     const bool dead = col_width == 0;
-    char* row = p.dq + ((int64_t)b * p.dq_sb + (int64_t)head * p.dq_sh + (int64_t)qrow * p.dq_ss) * 2;
+    __syncthreads();  // every wavefront has read its last tile
+    constexpr int kRowBytes = D * 2, kChunks = kRowBytes / 16, kRowsPerStore = 64 / kChunks;
+    char* stage = smem + wave * (32 * kRowBytes);
+    char* mine = stage + c * kRowBytes;
 #pragma unroll
     for (int dt = 0; dt < DT; dt++)
 #pragma unroll
@@ -363,8 +369,16 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_bwd_dq_kernel(const BwdParams
         u.x = Tr::pack2(dq[dt][4 * g4 + 0] * p.scale, dq[dt][4 * g4 + 1] * p.scale);
         u.y = Tr::pack2(dq[dt][4 * g4 + 2] * p.scale, dq[dt][4 * g4 + 3] * p.scale);
         if (dead) u = make_uint2(0, 0);
-        *reinterpret_cast<uint2*>(row + (32 * dt + 8 * g4 + 4 * h) * 2) = u;
+        *reinterpret_cast<uint2*>(mine + (((4 * dt + g4) ^ (c & (kChunks - 1))) * 16) + 8 * h) = u;
       }
+    char* dq0 = p.dq + ((int64_t)b * p.dq_sb + (int64_t)head * p.dq_sh) * 2;
+#pragma unroll
+    for (int r0 = 0; r0 < 32; r0 += kRowsPerStore) {
+      const int row = r0 + lane / kChunks, chunk = lane % kChunks;
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + row * kRowBytes + ((chunk ^ (row & (kChunks - 1))) * 16));
+      const int qr = q0 + wave * 32 + row;
+      if (qr < p.q_len) *reinterpret_cast<uint4*>(dq0 + (int64_t)qr * p.dq_ss * 2 + chunk * 16) = v;
+    }
   }
 }
 

@@ -506,6 +506,37 @@ __global__ __launch_bounds__(NW * 64, WPS) void fa_fwd_kernel(const FwdParams p)
   }
 
   // ---- epilogue: normalise, write O (query dtype) and lse --------------------------------
+  if constexpr (!SPLIT && MQ == 1) {
+    // A lane holds 4 consecutive head-dim elements of its query row per register group, so storing
+    // from the registers would touch 32 rows with 8 bytes each per instruction.  Each wavefront
+    // passes its 32 x D tile through its own part of the LDS (the tiles are done with) and writes
+    // whole rows, 16 bytes per lane; rows are swizzled by the row index against bank conflicts.
+    const float l = l_run[0] + xor32(l_run[0]);
+    const bool alive = l > 0.f && col_width[0] > 0;  // padding / out-of-range rows stay zero
+    const float inv = alive ? 1.f / l : 0.f;
+    if (row_in[0] && h == 0) lse[qrow[0]] = alive ? m_run[0] + fast_log2(l) : 0.f;
+    __syncthreads();  // every wavefront has read its last tile
+    constexpr int kRowBytes = D * 2, kChunks = kRowBytes / 16, kRowsPerStore = 64 / kChunks;
+    char* stage = smem + wave * (32 * kRowBytes);
+    char* mine = stage + c * kRowBytes;
+#pragma unroll
+    for (int dt = 0; dt < DTO; dt++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        uint2 u;
+        u.x = Tr::pack2(o[dt][0][4 * g4 + 0] * inv, o[dt][0][4 * g4 + 1] * inv);
+        u.y = Tr::pack2(o[dt][0][4 * g4 + 2] * inv, o[dt][0][4 * g4 + 3] * inv);
+        *reinterpret_cast<uint2*>(mine + (((4 * dt + g4) ^ (c & (kChunks - 1))) * 16) + 8 * h) = u;
+      }
+#pragma unroll
+    for (int r0 = 0; r0 < 32; r0 += kRowsPerStore) {
+      const int row = r0 + lane / kChunks, chunk = lane % kChunks;
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + row * kRowBytes + ((chunk ^ (row & (kChunks - 1))) * 16));
+      const int qr = q0 + wave * 32 + row;
+      if (qr < p.q_len) *reinterpret_cast<uint4*>(obase + (int64_t)qr * p.o_ss * 2 + chunk * 16) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int qt = 0; qt < MQ; qt++) {
     const float l = l_run[qt] + xor32(l_run[qt]);
