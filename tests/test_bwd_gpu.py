@@ -242,6 +242,29 @@ def test_positions_restart_per_document(device):
     check_all((dq, dk, dv), oracle_backward(data, w.scale, dout), data[4], data[6])
 
 
+@pytest.mark.parametrize("batch, hkv", [(1, 2), (3, 1), (3, 4), (5, 2)])
+def test_every_way_of_dealing_items_to_the_xcds(device, batch, hkv):
+    """(batch x kv heads) = 2, 3, 12 and 10 groups: groups shared between XCDs, groups cut into runs,
+    more than one group per XCD with some XCDs one short - the three ways the kernels deal their
+    work items out, with enough kv rows (18 items of 128 per group) for the dK/dV items to be ordered
+    by work, taken from queues and, the trailing padding ones, zero-filled without bookkeeping."""
+    s = 2304
+    lengths = generate_random_segments_lengths(s - 400, 5)
+    data, scale = make_random_attention_inputs(batch, s, s, 2 * hkv, hkv, 64, 64, seed=40 + batch + hkv,
+                                               num_pad_tokens=400, list_of_segment_lengths=lengths,
+                                               device=device)
+    dout = torch.randn(data[0].shape, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(device)
+    out, dq, dk, dv = run_backward(data, scale, (128, 128), (128, 128), dout)
+    q, k, v, *ids = [x.cpu() for x in data]
+    ref_out, _ = ao.attention_forward(q.float().numpy(), k.float().numpy(), v.float().numpy(),
+                                      *[i.numpy() for i in ids], scale)
+    check_grad("out", out, ref_out)
+    check_all((dq, dk, dv), oracle_backward(data, scale, dout), data[4], data[6])
+    dk32, dv32 = fp32_dkdv(data, scale, (128, 128), (128, 128), dout)
+    kpad = data[6].cpu().numpy() == -1
+    assert (dk32.cpu().numpy()[kpad] == 0).all() and (dv32.cpu().numpy()[kpad] == 0).all()
+
+
 def test_gqa_equals_repeated_kv_heads(device):
     data, scale = make_random_attention_inputs(1, 256, 256, 8, 2, 128, 128, seed=9, device=device)
     q, k, v, *ids = data
