@@ -454,30 +454,13 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   const bool p_wave = wave < NP;  // role, wave-uniform
 
   // The launch is one work-group per compute unit, and each takes work items (128 kv rows of one
-  // batch row and kv head) from the queue of its XCD until none is left: item j of XCD x is what
-  // work-group 8 j + x of a launch with one work-group per item would be.  (The hardware deals the
-  // work-groups of a launch to an XCD's four shader engines in strict rotation and in order, so a
-  // compute unit that finishes a long work-group waits until the rotation comes round to its
-  // engine: measured 6 to 12 % of this kernel's compute-unit time idle between work-groups.)  The
-  // index of the next item is requested when the current one's step loop has ended, so that its
-  // latency hides behind the final stores and an item is never held back by a long one.  A
-  // work-group whose XCD has run out of items takes them from the other XCDs' queues (the XCDs do
-  // not run at exactly the same speed): that costs L2 sharing, but only at the end of the launch.
+  // batch row and kv head) from the queues (see ItemQueue) until none is left.  The ticket for the
+  // next item is drawn when the current one's step loop has ended, so that its latency hides behind
+  // the final stores and an item is never held back by a long one.
   const ItemMap items{p.batch * p.num_kv_heads, p.num_tiles, 1};
-  int queue = blockIdx.x % 8;  // the queue this work-group currently draws from (thread 0 only)
-  // thread 0: the launch-wide index of the item that `ticket` of the current queue stands for, moving
-  // on to the next queue while the current one is exhausted; -1 when all are
-  auto resolve = [&](int ticket) {
-    for (int tries = 0;; tries++) {
-      const int id = 8 * ticket + queue;
-      if (id < p.total_items) return id;
-      if (tries == 7) return -1;
-      queue = (queue + 1) % 8;
-      ticket = atomicAdd(p.dkdv_queue + queue, 1);
-    }
-  };
+  ItemQueue work{p.dkdv_queue, p.total_items, (int)(blockIdx.x % 8)};  // thread 0's
   int* next_item = reinterpret_cast<int*>(smem + Smem::kTotal) + 1;
-  if (tid == 0) *next_item = resolve(atomicAdd(p.dkdv_queue + queue, 1));
+  if (tid == 0) *next_item = work.resolve(work.draw());
   __syncthreads();
   for (int item = *next_item; item >= 0; item = *next_item) {
   __syncthreads();  // every wavefront has read next_item
@@ -493,7 +476,7 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   const int k0 = kv_tile * TKV;
   if (entry & kDeadItem) {
     // no query tile can interact with these kv rows (known from the ordering pass): zeros, no bookkeeping
-    if (tid == 0) ticket = atomicAdd(p.dkdv_queue + queue, 1);
+    if (tid == 0) ticket = work.draw();
     const int row_bytes = D * (p.dkdv_f32 ? 4 : 2), chunks = row_bytes / 16;
     const int rows = min(TKV, p.kv_len - k0);
     for (int i = tid; i < rows * chunks; i += NW * 64) {
@@ -808,7 +791,7 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   __syncthreads();  // the next chunk reuses the bookkeeping, the rings and the exchange slots
   }
 
-  if (tid == 0) ticket = atomicAdd(p.dkdv_queue + queue, 1);
+  if (tid == 0) ticket = work.draw();
   // ---- epilogue: the P wave holds dV^T, the S wave dK^T (times the scale) ----------------------
   // A lane holds 4 consecutive head-dim elements of its kv row per register group, so storing from
   // the registers would touch 32 rows with 8 or 16 bytes each per instruction.  Each wavefront
@@ -868,9 +851,9 @@ __global__ __launch_bounds__(DkdvCfg<D>::kWaves * 64, DkdvCfg<D>::kWps) void fa_
   }
   }  // the item has work
   } else if (tid == 0) {
-    ticket = atomicAdd(p.dkdv_queue + queue, 1);
+    ticket = work.draw();
   }
-  if (tid == 0) *next_item = resolve(ticket);
+  if (tid == 0) *next_item = work.resolve(ticket);
   __syncthreads();
   }  // items of this XCD
 }
