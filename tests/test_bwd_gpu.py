@@ -79,11 +79,11 @@ def check_grad(name, got, ref, atol=ATOL, rel=0.0):
     return worst
 
 
-def check_all(grads, refs, q_seg, kv_seg, kv_atol=ATOL):
+def check_all(grads, refs, q_seg, kv_seg, kv_atol=ATOL, kv_rel=0.0):
     dq, dk, dv = grads
     check_grad("dq", dq, refs[0])
-    check_grad("dk", dk, refs[1], kv_atol)
-    check_grad("dv", dv, refs[2], kv_atol)
+    check_grad("dk", dk, refs[1], kv_atol, kv_rel)
+    check_grad("dv", dv, refs[2], kv_atol, kv_rel)
     qpad = q_seg.cpu().numpy() == -1
     kpad = kv_seg.cpu().numpy() == -1
     assert (dq.float().cpu().numpy()[qpad] == 0).all(), "padding rows of dQ must be zero"
@@ -431,6 +431,20 @@ def _random_case(seed, head_dim=None):
 # per dK/dV work-group, two steps per 64-row query tile, GQA groups up to 8)
 @pytest.mark.parametrize("seed, head_dim", [(i, None) for i in range(16)] + [(100 + i, 256) for i in range(8)])
 def test_randomized_shapes_forward_and_backward(device, seed, head_dim):
+    _check_random_case(device, seed, head_dim)
+
+
+def test_random_case_beyond_the_plain_bound(device):
+    """Of 184 further seeds (16-199, every fifth at head_dim 256) run once against the oracle, 183 met
+    the bounds of the test above and this one did not: one dK element of 3.28 came out as 3.3125,
+    2.92e-2 off where 2e-2 + half a bf16 ulp allows 2.78e-2 (second token of a 59-token document behind
+    462 padding tokens, GQA 4, head_dim 64; |dK| up to 8.8).  It is the rounding of dS to bf16 in
+    front of dS^T Q, which the reference prescribes (see tests/tolerances.py): the case is held to
+    the bound that carries that term."""
+    _check_random_case(device, 98, None, kv_rel=OPERAND_ROUNDING)
+
+
+def _check_random_case(device, seed, head_dim, kv_rel=0.0):
     c = _random_case(seed, head_dim)
     data, scale = make_random_attention_inputs(c["batch"], c["sq"], c["sk"], c["hq"], c["hkv"], c["d"], c["d"],
                                                seed=seed, num_pad_tokens=c["pad"],
@@ -464,6 +478,7 @@ def test_randomized_shapes_forward_and_backward(device, seed, head_dim):
                                       *[x.numpy() for x in ids_], scale)
     assert np.abs(out.float().cpu().numpy() - ref_out).max() <= ATOL, c
     refs = oracle_backward(data, scale, dout)
-    check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if c["hq"] // c["hkv"] >= 8 else ATOL)
+    check_all((dq, dk, dv), refs, data[4], data[6], kv_atol=5e-2 if c["hq"] // c["hkv"] >= 8 else ATOL,
+              kv_rel=kv_rel)
     if c["hq"] // c["hkv"] >= 8:
         check_fp32_dkdv(data, scale, blocks, blocks, dout, refs)
