@@ -149,7 +149,8 @@ typedef struct kvax_fa_args {
  *             share one key sequence (a function of the shapes only), plus, with KVAX_FA_FWD_WIDE,
  *             the lists of live kv tiles per 256 query rows;
  *   backward: delta [batch, num_heads, q_len] fp32, the tile summaries of the kv and the query
- *             sequence, and the dispatch order of the dK/dV work items (longest first). */
+ *             sequence, the order in which the dK/dV kernel takes its work items and the counters of
+ *             the queues it takes them from (cleared by the call itself). */
 size_t kvax_fa_fwd_workspace_bytes(const kvax_fa_args* args);
 size_t kvax_fa_bwd_workspace_bytes(const kvax_fa_args* args);
 int kvax_fa_fwd(const kvax_fa_args* args, void* workspace, size_t workspace_bytes,
