@@ -38,6 +38,12 @@ def _as_ids(x: DeviceArray, name: str) -> torch.Tensor:
 
 _LAYOUTS: dict = {}
 
+try:  # the stream handle without building a torch.cuda.Stream object around it (4 us of a 27 us call)
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:  # pragma: no cover - older or newer torch without the private helper
+    def _raw_stream(index: int) -> int:
+        return torch.cuda.current_stream(index).cuda_stream
+
 
 def _layout(lib, batch, q_len, kv_len, requests, num_q_shards):
     """Where the masks of a call lie in its one allocation (in int32 words after the workspace), and
@@ -103,11 +109,21 @@ def build_masks(
         n = b * shards * n_outer
         first = base + 4 * (ws_words + off)
         d.lower, d.upper, d.lower_full, d.upper_full = first, first + 4 * n, first + 8 * n, first + 12 * n
-        views = buf[ws_words + off:ws_words + off + 4 * n].view(4, b, shards, n_outer).unbind(0)
-        masks.append(AttentionMask(*views))
-    stream = torch.cuda.current_stream(device).cuda_stream
+    _, b, shards, n_outer = shapes[0]
+    n4 = 4 * b * shards * n_outer
+    if n4 % 4 == 0 and all(sh[1:] == shapes[0][1:] for sh in shapes):
+        # equal shapes lie back to back: one view of all of them and one unbind
+        flat = buf[ws_words:ws_words + len(shapes) * n4].view(len(shapes) * 4, b, shards, n_outer).unbind(0)
+        masks = [AttentionMask(*flat[4 * i:4 * i + 4]) for i in range(len(shapes))]
+    else:
+        for off, b, shards, n_outer in shapes:
+            n = b * shards * n_outer
+            views = buf[ws_words + off:ws_words + off + 4 * n].view(4, b, shards, n_outer).unbind(0)
+            masks.append(AttentionMask(*views))
     index = device.index
-    if index is None or index == torch.cuda.current_device():
+    current = torch.cuda.current_device()
+    stream = _raw_stream(current if index is None else index)
+    if index is None or index == current:
         rc = lib.kvax_mask_build(
             q_pos.data_ptr(), q_seg.data_ptr(), kv_pos.data_ptr(), kv_seg.data_ptr(),
             batch, q_len, kv_len, num_q_shards, int(skip_pad_tokens),
